@@ -1,0 +1,230 @@
+"""MicroAdam step benchmark on one MI355X.
+
+A "step" is one `optimizer.step()` over the whole parameter list of the workload, with
+parameters, gradients and optimizer state already resident in HBM.  The default workload is the
+Llama-2-7B-shaped list (6.74 B bf16 parameters, m=10, k=1 %, quant block 64, alpha=0).
+Gradients are synthetic N(0, 1e-3^2) bf16, drawn on the device before the timed region; a few
+distinct gradient sets are rotated so that consecutive steps see different data.
+
+Prints ONE JSON line: params/s (whole job), ms per step, the HBM roofline of the fused step
+kernel (algorithmic bytes per parameter x parameters / measured duration against 8 TB/s) and a
+CPU baseline: the C oracle (a port of the reference's step; the reference has no CPU path)
+timed on this host's cores over a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ista-daslab-optimizers_amd"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def llama2_7b():
+    shapes = [(32000, 4096)]
+    for _ in range(32):
+        shapes += [(4096, 4096)] * 4 + [(11008, 4096)] * 3 + [(4096,)] * 2
+    shapes += [(32000, 4096)]
+    return shapes
+
+
+def gpt2_small():
+    shapes = [(50257, 768), (1024, 768)]
+    for _ in range(12):
+        shapes += [(768,), (768,), (768, 2304), (2304,), (768, 768), (768,), (768,), (768,),
+                   (768, 3072), (3072,), (3072, 768), (768,)]
+    shapes += [(768,), (768,)]
+    return shapes
+
+
+def outlier_1p3b():
+    shapes = [(50304, 2048)]
+    for _ in range(24):
+        shapes += [(2048, 6144), (2048, 2048), (2048, 8192), (8192, 2048)]
+    return shapes
+
+
+def llama3_8b():
+    shapes = [(128256, 4096)]
+    for _ in range(32):
+        shapes += [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096)] + [(14336, 4096)] * 3
+    shapes += [(128256, 4096)]
+    return shapes
+
+
+WORKLOADS = {
+    # name: (shapes, dtype, m, k_init, q, alpha, grad_std)
+    "llama2-7b": (llama2_7b, "bf16", 10, 0.01, 64, 0.0, 1e-3),
+    "gpt2-small": (gpt2_small, "bf16", 10, 0.01, 64, 0.0, 1e-2),
+    "outlier-1.3b": (outlier_1p3b, "bf16", 20, 0.05, 32, 0.0, 1e-3),
+    "llama3-8b": (llama3_8b, "bf16", 10, 0.01, 100000, 0.5, 1e-3),
+    "plumbing-1m": (lambda: [(1048576,)], "f32", 10, 0.01, 64, 0.0, 1.0),
+}
+
+
+def numel(shape):
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+def algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, d_block_size, steps_done):
+    """Every array of the step touched once: read g, read+write 4-bit EF, read+write p, write
+    one window row (int16 + bf16), read min(t, m) window rows, read+write bf16 min/max."""
+    import math
+    s = 2 if dtype == "bf16" else 4
+    total_d = total_k = total_stats = 0
+    for shp in shapes:
+        d = numel(shp)
+        dbs = min(d, d_block_size)
+        full = d // dbs
+        k = full * math.ceil(dbs * k_init) + math.ceil((d - full * dbs) * k_init)
+        total_d += d
+        total_k += k
+        total_stats += (d + q - 1) // q
+    rows = min(steps_done, m)
+    b = total_d * (s + 0.5 + 0.5 + 2 * s) + total_k * 4 * (1 + rows) + total_stats * 8
+    if alpha > 0:
+        b += total_d * 1.0  # the EF is read and written a second time
+    return b / total_d
+
+
+def cpu_baseline(workload, budget_s=20.0):
+    """The C oracle on this host's cores, on a bounded sample of the workload."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import microadam_oracle as oracle
+    oracle.build()
+    shapes_fn, dtype, m, k_init, q, alpha, gstd = WORKLOADS[workload]
+    shapes = shapes_fn()
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    oracle.set_threads(cores)
+    # sample: the first tensors of one repeating layer, up to ~200 M parameters
+    sample, total = [], 0
+    for shp in shapes[1:]:
+        if total + numel(shp) > 210_000_000:
+            break
+        sample.append(shp)
+        total += numel(shp)
+    if not sample:
+        sample, total = [shapes[0]], numel(shapes[0])
+    rng = np.random.default_rng(0)
+
+    def draw(n, std):
+        x = rng.standard_normal(n, dtype=np.float32) * np.float32(std)
+        return oracle.f32_to_bf16(x) if dtype == "bf16" else x
+
+    params = [draw(numel(s), 0.02) for s in sample]
+    opt = oracle.OracleMicroAdam(params, m, 1e-3, q, k_init, alpha)
+    steps, elapsed = 0, 0.0
+    while steps < 1 or (elapsed < budget_s and steps < 3):
+        grads = [draw(numel(s), gstd) for s in sample]
+        t0 = time.perf_counter()
+        opt.step(grads)
+        elapsed += time.perf_counter() - t0
+        steps += 1
+    return {"value": total * steps / elapsed, "unit": "params/s", "cores": cores, "kind": "port",
+            "sample": f"{len(sample)} tensors ({total} params) of the {workload} list, "
+                      f"{steps} steps, C oracle with OpenMP"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--workload", default="llama2-7b", choices=sorted(WORKLOADS))
+    ap.add_argument("--grad-sets", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--op-by-op", action="store_true", help="time the unfused route instead")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
+
+    import torch
+    from ista_daslab_optimizers import MicroAdam
+
+    shapes_fn, dtype, m, k_init, q, alpha, gstd = WORKLOADS[args.workload]
+    shapes = shapes_fn()
+    tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    params = []
+    for shp in shapes:
+        p = torch.empty(shp, dtype=tdtype, device=dev)
+        p.normal_(0, 0.02)
+        params.append(torch.nn.Parameter(p))
+    n_params = sum(p.numel() for p in params)
+    grad_sets = []
+    for _ in range(max(1, args.grad_sets)):
+        gs = []
+        for shp in shapes:
+            g = torch.empty(shp, dtype=tdtype, device=dev)
+            g.normal_(0, gstd)
+            gs.append(g)
+        grad_sets.append(gs)
+
+    opt = MicroAdam(params, m=m, lr=1e-3, quant_block_size=q, k_init=k_init, alpha=alpha,
+                    betas=(0.9, 0.999), eps=1e-8, weight_decay=0)
+    opt.use_fused = not args.op_by_op
+
+    def one_step(i):
+        gs = grad_sets[i % len(grad_sets)]
+        for p, g in zip(params, gs):
+            p.grad = g
+        opt.step()
+
+    for i in range(args.warmup):
+        one_step(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        one_step(args.warmup + i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = sorted(a.elapsed_time(b) for a, b in ev)
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_ms = sum(dev_ms) / len(dev_ms)
+
+    bpp = algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, opt.d_block_size,
+                                      args.warmup + args.steps)
+    achieved = bpp * n_params / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "MicroAdam step throughput (params/s) at the Llama-2-7B shape"
+                  if args.workload == "llama2-7b" else f"MicroAdam step throughput ({args.workload})",
+        "value": n_params / (ms_per_step * 1e-3),
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {"workload": args.workload, "params": n_params, "tensors": len(shapes), "m": m,
+                   "k_init": k_init, "quant_block_size": q, "alpha": alpha,
+                   "d_block_size": opt.d_block_size,
+                   "route": "op-by-op" if args.op_by_op else "fused"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
+                     "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},
+    }
+    if not args.no_cpu_baseline:
+        del grad_sets
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

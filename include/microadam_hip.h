@@ -1,0 +1,167 @@
+/*
+ * C ABI of libmicroadam_hip.so: the MicroAdam optimizer step as gfx950 HIP kernels.
+ *
+ * The reference (IST-DASLab/ISTA-DASLab-Optimizers) reaches its device code through two
+ * pybind extension modules of the separate package ista-daslab-optimizers-cuda
+ * (pyproject.toml:21): ista_daslab_cuda_tools and ista_daslab_cuda_micro_adam.  Every
+ * function those modules export on the MicroAdam path has one entry point here with the
+ * same argument order and meaning; the call sites cited below are in
+ * ista_daslab_optimizers/micro_adam/micro_adam.py (MA) and ista_daslab_optimizers/tools.py.
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers unless a comment says "host".
+ *  - dtype: MA_F32 (0) = float, MA_BF16 (1) = bfloat16 bit patterns (uint16_t).  It is the
+ *    type of the dense vectors (gradient / accumulator / update / parameter).  Window values,
+ *    and the per-block min / max statistics, are always bf16; window indices int16; error
+ *    feedback is packed 4-bit codes, element 2j in the high nibble of byte j.
+ *  - stream: a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued and
+ *    the call returns; nothing here synchronises, allocates or frees device memory.
+ *  - Return value: 0 on success; a positive hipError_t if the runtime refused a launch; a
+ *    negative MA_ERR_* code if the arguments are rejected before anything is launched.
+ *  - Arithmetic: fp32, no fused multiply-add, round-to-nearest-even into the destination type.
+ */
+#ifndef MICROADAM_HIP_H
+#define MICROADAM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MA_F32 0
+#define MA_BF16 1
+
+#define MA_ERR_ARG (-1)         /* null pointer, non-positive size, unknown dtype / direction */
+#define MA_ERR_BLOCK_SIZE (-2)  /* top-k block longer than 32768 (int16 indices) */
+#define MA_ERR_WINDOW (-3)      /* m larger than MA_MAX_WINDOW */
+#define MA_ERR_GEOMETRY (-4)    /* k / k_block_size inconsistent with d and d_block_size */
+#define MA_ERR_NOT_FUSABLE (-5) /* tensor does not meet ma_fused_step's layout conditions */
+#define MA_ERR_LDS (-6)         /* the launch would need more than 160 KB of LDS */
+
+#define MA_MAX_WINDOW 64 /* largest window length m the kernels take */
+#define MA_MAX_D_BLOCK 32768
+
+const char *ma_error_string(int code);
+
+/* ---- ista_daslab_cuda_tools ------------------------------------------------------------ */
+
+/* get_sm_count(), MA:40: compute units of the current device (256 on MI355X). */
+int ma_get_sm_count(void);
+
+/* get_max_floats_for_shared_memory_per_thread_block(), MA:43: fp32 slots of LDS one
+ * workgroup may use, 160 KB / 4 = 40960 on gfx950; MA:44 halves it into d_block_size. */
+int ma_get_max_floats_for_shared_memory_per_thread_block(void);
+
+/* copy_values(d, k, d_block_size, k_block_size, indices, inp, out, direction), MA:202-209.
+ * direction 1 (d2k): out[j] = bf16(inp[(j / k_block_size) * d_block_size + indices[j]]),
+ *   inp is `dtype` of length d, out is bf16 of length k.
+ * direction 0 (k2d, sparse_mfac/sparse_core_mfac_w_ef.py:117-124): the reverse scatter,
+ *   inp is bf16 of length k, out is `dtype` of length d. */
+int ma_copy_values(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
+                   const int16_t *indices, const void *inp, void *out, int direction, int dtype,
+                   void *stream);
+
+/* zerorize_block_components(vector, indices, d, k, d_block_size, k_block_size), MA:214:
+ * vector[(j / k_block_size) * d_block_size + indices[j]] = 0. */
+int ma_zerorize_block_components(void *vector, const int16_t *indices, int64_t d, int64_t k,
+                                 int64_t d_block_size, int64_t k_block_size, int dtype,
+                                 void *stream);
+
+/* ---- ista_daslab_cuda_micro_adam --------------------------------------------------------- */
+
+/* asymm_block_quant(d, q_block_size, xq, xmin, xmax, x), MA:231, MA:316:
+ * xq = Q(x): code = clamp(floor((x - min_b) / u_b + 0.5), 0, 15), u_b = (max_b - min_b) / 15,
+ * b = i / q_block_size; a zero or non-finite range gives code 0. */
+int ma_asymm_block_quant(int64_t d, int64_t q_block_size, uint8_t *xq, const uint16_t *xmin,
+                         const uint16_t *xmax, const void *x, int dtype, void *stream);
+
+/* asymm_block_quant_inv(d, q_block_size, xq, xmin, xmax, x, alpha), MA:190, :267, :298, :313,
+ * :322: x += alpha * (code * u_b + min_b). */
+int ma_asymm_block_quant_inv(int64_t d, int64_t q_block_size, const uint8_t *xq,
+                             const uint16_t *xmin, const uint16_t *xmax, void *x, float alpha,
+                             int dtype, void *stream);
+
+/* compute_microadam_update(blocks, threads, carveout, t, beta1, beta2, eps, d_block_size,
+ * k_block_size, d, m, k, indices, values, out), MA:277-291.  For every coordinate named by a
+ * live window row (row i < min(t, m), age (t-1-i) mod m): z1 = sum beta1^age v, z2 = sum
+ * beta2^age v^2 in increasing row order, out = (z1 s1) / (eps + sqrt(z2 s2)) with
+ * s = (1-beta)/(1-beta^t).  Entries whose value is +-0 are skipped; coordinates no other entry
+ * names are left as they are (the caller zeroes out first, MA:276).  blocks / threads / carveout are the reference's launch hints; they
+ * are accepted and ignored (one workgroup per top-k block is launched). */
+int ma_compute_microadam_update(int blocks, int threads, int carveout, int64_t t, double beta1,
+                                double beta2, double eps, int64_t d_block_size,
+                                int64_t k_block_size, int64_t d, int64_t m, int64_t k,
+                                const int16_t *indices, const uint16_t *values, void *out,
+                                int dtype, void *stream);
+
+/* ---- stock torch ops of the hot path, as kernels ------------------------------------------ */
+
+/* Replaces torch.abs + torch.topk + .to(int16) + slice assignment, MA:193-200, and optionally
+ * MA:202-209 and MA:214 in the same launch.  For every top-k block of x (d_block_size
+ * elements, the last one shorter) the k_block entries largest in magnitude are found, exact
+ * ties at the threshold going to the lowest indices; I_row receives their block-relative
+ * indices in ascending order (k_many per full block, then k_few for the tail block).
+ * V_row, if not NULL, receives bf16(x) at those positions; if zero_selected != 0 they are
+ * then set to 0 in x. */
+int ma_block_topk(int64_t d, int64_t d_block_size, int64_t k_many, int64_t k_few, void *x,
+                  int16_t *I_row, uint16_t *V_row, int zero_selected, int dtype, void *stream);
+
+/* Replaces _update_quantization_statistics, MA:217-228: bf16 min and max of every
+ * quantisation block [b*q, min((b+1)*q, d)) of x. */
+int ma_block_minmax(int64_t d, int64_t q_block_size, const void *x, uint16_t *xmin,
+                    uint16_t *xmax, int dtype, void *stream);
+
+/* Replaces p.mul_(1 - lr*wd) (MA:234-235, skipped when apply_decay == 0) followed by
+ * p.add_(u, alpha=-lr) (MA:304): p = rne(p * decay); p = rne(p + neg_lr * u). */
+int ma_param_update(int64_t d, void *p, const void *u, float neg_lr, int apply_decay,
+                    float decay, int dtype, void *stream);
+
+/* ---- the fused step ------------------------------------------------------------------------ */
+
+/* One parameter tensor of a fused step.  Pointers are device pointers; the struct itself is
+ * host memory. */
+typedef struct ma_tensor {
+    void *p;            /* parameter, `dtype`, d elements */
+    void *g;            /* gradient, `dtype`, d elements; NOT modified by the fused step */
+    uint8_t *error;     /* st['error'],    ceil(d/2) bytes,            MA:92 */
+    uint16_t *min_vals; /* st['min_vals'], quant_full_blocks_count+1,  MA:93 */
+    uint16_t *max_vals; /* st['max_vals'],                             MA:94 */
+    int16_t *I;         /* st['I'], m x k,                             MA:86 */
+    uint16_t *V;        /* st['V'], m x k,                             MA:87 */
+    int64_t d;          /* st['d'] */
+    int64_t k;          /* st['k'], row length of I and V,             MA:82 */
+    double lr;          /* group['lr'],                                MA:121 */
+    double weight_decay; /* group['weight_decay'],                     MA:122 */
+    int32_t index;      /* st['index'], the ring row written by this step, MA:180 */
+    int32_t reserved;
+} ma_tensor;
+
+typedef struct ma_hyper {
+    int64_t t;          /* self.steps after the increment, MA:98, :280 */
+    int32_t m;          /* window length */
+    int32_t dtype;      /* MA_F32 or MA_BF16, of p and g */
+    int64_t quant_block_size;
+    int64_t d_block_size; /* self.d_block_size, MA:44 */
+    double k_init;
+    double beta1, beta2, eps;
+} ma_hyper;
+
+/* The whole of update_step (MA:146-328) for alpha == 0, for a list of tensors, in one pass per
+ * top-k block: a = g + Qinv(e); block top-k -> I[index], V[index]; residual -> new min/max
+ * and 4-bit codes; window -> Adam direction; p update (with decoupled weight decay).  The
+ * caller advances st['index'] (MA:211) itself.  Conditions (else MA_ERR_NOT_FUSABLE, nothing
+ * launched): quant_block_size a power of two in [8, 512] that divides d_block_size (or
+ * d <= d_block_size) and does not exceed d; p and g 16-byte aligned, error 4-byte aligned;
+ * d_block_size a multiple of 8 unless d <= d_block_size. */
+int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
+                  const ma_hyper *hyper /* host */, void *stream);
+
+/* 0 if ma_fused_step would accept this tensor under `hyper`, else the MA_ERR_* it would
+ * return.  Host-only check, launches nothing. */
+int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,397 @@
+// Device-side building blocks of the MicroAdam step for gfx950 (wave64, 160 KB LDS per CU).
+//
+// One workgroup of 256 threads (4 waves, one per SIMD) owns one top-k block of up to
+// 2048*C elements and keeps it in VGPRs for the whole step.  Wave w, chunk c, lane l holds
+// the 8 consecutive elements starting at ((w*C + c)*64 + l)*8, so every 128-bit load of a
+// wave covers one contiguous KiB (bf16) and the block's index order is (wave, chunk, lane,
+// element).  Elements past the block's length read as +0.0, which the lowest-index tie rule
+// makes harmless for the selection: a padded zero can never rank before a real element.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ma {
+
+constexpr int kWG = 256;
+constexpr int kWave = 64;
+constexpr int kWaves = kWG / kWave;
+constexpr int kChunk = 8;        // elements per lane per chunk
+constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
+constexpr int kMaxWindow = 64;
+
+// ---- scalar helpers -----------------------------------------------------------------------
+
+__device__ __forceinline__ float bf2f(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t f2bf(float f) {
+    __bf16 b = (__bf16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+
+__device__ __forceinline__ uint32_t f2bf_pair(float lo, float hi) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    f2 v = {lo, hi};
+    b2 r = __builtin_convertvector(v, b2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ uint32_t mbcnt(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        uint32_t t = __shfl_up(v, d, kWave);
+        if (lane >= d) v += t;
+    }
+    return v;
+}
+
+// Inclusive scan over the 256 threads in thread order.  sh4 is 4 words of LDS.
+__device__ __forceinline__ uint32_t wg_incl_scan(uint32_t v, uint32_t *sh4, int lane, int wave) {
+    uint32_t s = wave_incl_scan(v, lane);
+    if (lane == kWave - 1) sh4[wave] = s;
+    __syncthreads();
+    uint32_t add = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+        if (w < wave) add += sh4[w];
+    __syncthreads();
+    return s + add;
+}
+
+// ---- a top-k block in registers ------------------------------------------------------------
+
+template <int C>
+struct RegsBF16 {
+    static constexpr int kC = C;
+    static constexpr bool kBF16 = true;
+    static constexpr int kElemBytes = 2;
+    typedef uint16_t elem_t;
+    typedef uint16_t slot_t;  // LDS cell that first holds a slot id, later the update's bits
+    uint32_t w[C][4];         // two bf16 per register
+
+    __device__ __forceinline__ uint32_t key(int c, int e) const {
+        uint32_t x = w[c][e >> 1];
+        return (e & 1) ? ((x >> 16) & 0x7fffu) : (x & 0x7fffu);
+    }
+    __device__ __forceinline__ float val(int c, int e) const {
+        uint32_t x = w[c][e >> 1];
+        return __uint_as_float((e & 1) ? (x & 0xffff0000u) : (x << 16));
+    }
+    __device__ __forceinline__ uint32_t bf16_bits(int c, int e) const {
+        uint32_t x = w[c][e >> 1];
+        return (e & 1) ? (x >> 16) : (x & 0xffffu);
+    }
+    __device__ __forceinline__ void zero(int c, int e) {
+        w[c][e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+    }
+    __device__ __forceinline__ void set_chunk(int c, const float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[c][i] = f2bf_pair(v[2 * i], v[2 * i + 1]);
+    }
+};
+
+template <int C>
+struct RegsF32 {
+    static constexpr int kC = C;
+    static constexpr bool kBF16 = false;
+    static constexpr int kElemBytes = 4;
+    typedef float elem_t;
+    typedef uint32_t slot_t;
+    float w[C][8];
+
+    __device__ __forceinline__ uint32_t key(int c, int e) const {
+        return __float_as_uint(w[c][e]) & 0x7fffffffu;
+    }
+    __device__ __forceinline__ float val(int c, int e) const { return w[c][e]; }
+    __device__ __forceinline__ uint32_t bf16_bits(int c, int e) const { return f2bf(w[c][e]); }
+    __device__ __forceinline__ void zero(int c, int e) { w[c][e] = 0.0f; }
+    __device__ __forceinline__ void set_chunk(int c, const float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[c][i] = v[i];
+    }
+};
+
+// element offset of (wave, chunk, lane) inside the block
+template <int C>
+__device__ __forceinline__ int chunk_off(int wave, int c, int lane) {
+    return ((wave * C + c) * kWave + lane) * kChunk;
+}
+
+// Load 8 consecutive elements as fp32.  `vec` says the 16-byte path is legal for this block
+// (base 16-byte aligned); chunks that cross the block's end go element by element and
+// elements past `n` read as +0.0.
+__device__ __forceinline__ void load8(const uint16_t *base, int off, int n, bool vec,
+                                      float (&v)[8]) {
+    if (vec && off + kChunk <= n) {
+        uint4 q = *reinterpret_cast<const uint4 *>(base + off);
+        uint32_t r[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(r[i] << 16);
+            v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (off + i < n) ? bf2f(base[off + i]) : 0.0f;
+    }
+}
+
+__device__ __forceinline__ void load8(const float *base, int off, int n, bool vec,
+                                      float (&v)[8]) {
+    if (vec && off + kChunk <= n) {
+        float4 a = *reinterpret_cast<const float4 *>(base + off);
+        float4 b = *reinterpret_cast<const float4 *>(base + off + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (off + i < n) ? base[off + i] : 0.0f;
+    }
+}
+
+// Store 8 consecutive elements given as fp32, rounding to the element type.
+__device__ __forceinline__ void store8(uint16_t *base, int off, int n, bool vec,
+                                       const float (&v)[8]) {
+    if (vec && off + kChunk <= n) {
+        uint4 q;
+        q.x = f2bf_pair(v[0], v[1]);
+        q.y = f2bf_pair(v[2], v[3]);
+        q.z = f2bf_pair(v[4], v[5]);
+        q.w = f2bf_pair(v[6], v[7]);
+        *reinterpret_cast<uint4 *>(base + off) = q;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (off + i < n) base[off + i] = (uint16_t)f2bf(v[i]);
+    }
+}
+
+__device__ __forceinline__ void store8(float *base, int off, int n, bool vec,
+                                       const float (&v)[8]) {
+    if (vec && off + kChunk <= n) {
+        *reinterpret_cast<float4 *>(base + off) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(base + off + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (off + i < n) base[off + i] = v[i];
+    }
+}
+
+template <class R>
+__device__ __forceinline__ void load_block(R &r, const typename R::elem_t *base, int n, bool vec,
+                                           int wave, int lane) {
+#pragma unroll
+    for (int c = 0; c < R::kC; ++c) {
+        float v[8];
+        load8(base, chunk_off<R::kC>(wave, c, lane), n, vec, v);
+        r.set_chunk(c, v);
+    }
+}
+
+// ---- threshold search: MSD radix select over the magnitude bits -----------------------------
+//
+// Finds the key T of the kb-th largest magnitude and how many entries equal to T belong to
+// the top kb (`take_eq` >= 1).  Each pass histograms one digit of the keys that still match
+// the prefix into `hist`, 32 replicated copies per bin so that every lane adds into its own
+// LDS bank whatever the data look like, then scans the bins from the top.
+//   hist: 256*32 words, sh: 8 words.  Ends with a barrier.
+template <class R>
+__device__ __forceinline__ void select_threshold(const R &r, int kb, uint32_t *hist, uint32_t *sh,
+                                                 uint32_t &T, int &take_eq) {
+    constexpr int kPasses = R::kBF16 ? 2 : 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t prefix = 0, pmask = 0;
+    int need = kb;
+#pragma unroll
+    for (int pass = 0; pass < kPasses; ++pass) {
+        const int bits = (pass == kPasses - 1) ? 7 : 8;
+        const int shift = R::kBF16 ? (pass == 0 ? 7 : 0) : (pass == 3 ? 0 : 23 - 8 * pass);
+        const int nb = 1 << bits;
+        const uint32_t dm = nb - 1;
+        for (int i = tid; i < nb * kHistCopies / 4; i += kWG)
+            reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < R::kC; ++c) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                uint32_t key = r.key(c, e);
+                if ((key & pmask) == prefix)
+                    atomicAdd(&hist[(((key >> shift) & dm) << 5) + (lane & 31)], 1u);
+            }
+        }
+        __syncthreads();
+        // thread tid owns bin nb-1-tid so that a forward scan walks the bins from the top
+        const int bin = nb - 1 - tid;
+        uint32_t cnt = 0;
+        if (bin >= 0) {
+#pragma unroll 8
+            for (int j = 0; j < kHistCopies; ++j) cnt += hist[(bin << 5) + ((j + tid) & 31)];
+        }
+        uint32_t incl = wg_incl_scan(cnt, sh, lane, wave);
+        uint32_t excl = incl - cnt;
+        if (bin >= 0 && excl < (uint32_t)need && (uint32_t)need <= incl) {
+            sh[4] = (uint32_t)bin;
+            sh[5] = (uint32_t)need - excl;
+        }
+        __syncthreads();
+        prefix |= sh[4] << shift;
+        pmask |= dm << shift;
+        need = (int)sh[5];
+    }
+    __syncthreads();
+    T = prefix;
+    take_eq = need;
+}
+
+// ---- ordered compaction ------------------------------------------------------------------------
+//
+// Selects every entry with key > T plus the first `take_eq` entries (in index order) with
+// key == T, writes (block-relative index, bf16 value) to sel_idx / sel_val in ascending index
+// order and zeroes the selected entries in the registers.  sh: 8 words.  Ends with a barrier.
+template <class R>
+__device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, int kb,
+                                                 uint16_t *sel_idx, uint16_t *sel_val,
+                                                 uint32_t *sh) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t pre[R::kC];  // low 16: entries >= T before this lane's chunk; high 16: == T
+    uint32_t run = 0;
+#pragma unroll
+    for (int c = 0; c < R::kC; ++c) {
+        uint32_t cnt = 0;
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            uint32_t key = r.key(c, e);
+            cnt += (key >= T ? 1u : 0u) + (key == T ? 0x10000u : 0u);
+        }
+        uint32_t incl = wave_incl_scan(cnt, lane);
+        pre[c] = run + incl - cnt;
+        run += __shfl(incl, kWave - 1, kWave);
+    }
+    if (lane == 0) sh[wave] = run;
+    __syncthreads();
+    uint32_t base = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+        if (w < wave) base += sh[w];
+#pragma unroll
+    for (int c = 0; c < R::kC; ++c) {
+        uint32_t p = pre[c] + base;
+        uint32_t ge_before = p & 0xffffu, eq_before = p >> 16;
+        const int off = chunk_off<R::kC>(wave, c, lane);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            uint32_t key = r.key(c, e);
+            if (key >= T) {
+                bool is_eq = key == T;
+                bool sel = !is_eq || eq_before < (uint32_t)take_eq;
+                uint32_t pos = (ge_before - eq_before) + min(eq_before, (uint32_t)take_eq);
+                if (sel && pos < (uint32_t)kb) {
+                    sel_idx[pos] = (uint16_t)(off + e);
+                    sel_val[pos] = (uint16_t)r.bf16_bits(c, e);
+                    r.zero(c, e);
+                }
+                ge_before += 1;
+                eq_before += is_eq ? 1u : 0u;
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// ---- Adam statistics of one block from its window rows ---------------------------------------------
+//
+// slot[i] (one cell per block coordinate, zeroed by the caller) maps a coordinate to 1 + its
+// row in z1 / z2 / coord; rows are handed out on first touch.  Only coordinates in [lo, hi) are
+// considered, so a caller short of LDS can walk the block in several ranges.  Window rows are
+// visited in increasing row order with a barrier between rows, and inside a row all indices are
+// distinct, so every coordinate's sums are formed in a fixed order.  On return (after a
+// barrier) `*counter` holds the number of touched coordinates (at most `cap`), coord[s] their
+// block-relative index and z1[s], z2[s] the weighted sums.
+struct WindowView {
+    const int16_t *I;   // window indices, row stride k, already offset to this block's columns
+    const uint16_t *V;  // window values, same layout
+    int64_t k;
+    int rows;           // live rows: min(t, m)
+    int cur_row;        // row written in this step, taken from LDS instead of memory (-1: none)
+    const uint16_t *cur_idx;
+    const uint16_t *cur_val;
+    const float *w1;    // beta1^age per row
+    const float *w2;
+};
+
+template <typename slot_t>
+__device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, int lo, int hi,
+                                                  slot_t *slot, float *z1, float *z2,
+                                                  uint16_t *coord, uint32_t *counter, int cap) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    if (tid == 0) *counter = 0;
+    __syncthreads();
+    const int trips = (kb + kWG - 1) / kWG;
+    for (int row = 0; row < wv.rows; ++row) {
+        const float w1 = wv.w1[row], w2 = wv.w2[row];
+        for (int it = 0; it < trips; ++it) {
+            const int j = it * kWG + tid;
+            int idx = 0;
+            uint32_t vb = 0;
+            bool active = j < kb;
+            if (active) {
+                if (row == wv.cur_row) {
+                    idx = wv.cur_idx[j];
+                    vb = wv.cur_val[j];
+                } else {
+                    idx = wv.I[(int64_t)row * wv.k + j];
+                    vb = wv.V[(int64_t)row * wv.k + j];
+                }
+                // the range test also keeps a corrupt index from leaving the block; +-0 values
+                // add nothing and are skipped, which keeps the all-(0, 0) rows of a fresh
+                // window from naming coordinate 0 many times in one row
+                active = idx >= lo && idx < hi && (vb & 0x7fffu) != 0;
+            }
+            const float v = bf2f(vb);
+            const float a1 = w1 * v;
+            const float vv = v * v;
+            const float a2 = w2 * vv;
+            uint32_t s = active ? (uint32_t)slot[idx] : 1u;
+            const bool fresh = active && s == 0;
+            const uint64_t mask = __ballot(fresh);
+            if (mask != 0) {
+                const int leader = __ffsll((unsigned long long)mask) - 1;
+                uint32_t first = 0;
+                if (lane == leader) first = atomicAdd(counter, (uint32_t)__popcll(mask));
+                first = __shfl(first, leader, kWave);
+                if (fresh) {
+                    s = first + mbcnt(mask) + 1;
+                    if (s <= (uint32_t)cap) {  // always true for duplicate-free rows
+                        slot[idx] = (slot_t)s;
+                        coord[s - 1] = (uint16_t)idx;
+                        z1[s - 1] = 0.0f + a1;
+                        z2[s - 1] = 0.0f + a2;
+                    }
+                }
+            }
+            if (active && !fresh) {
+                z1[s - 1] = z1[s - 1] + a1;
+                z2[s - 1] = z2[s - 1] + a2;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ float adam_direction(float z1, float z2, float s1, float s2,
+                                                float eps) {
+    const float mh = z1 * s1;
+    const float vh = z2 * s2;
+    const float den = eps + sqrtf(vh);
+    return mh / den;
+}
+
+}  // namespace ma

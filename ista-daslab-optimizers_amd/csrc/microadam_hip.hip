@@ -1,0 +1,1009 @@
+// libmicroadam_hip.so: kernels, launchers and the C ABI declared in include/microadam_hip.h.
+// gfx950 only.  Built by csrc/Makefile with -ffp-contract=off so that the fp32 arithmetic is
+// the unfused sequence the header describes.
+#include "ma_device.hpp"
+
+#include <math.h>
+#include <string.h>
+
+#include "../../include/microadam_hip.h"
+
+namespace ma {
+
+// =============================================================================================
+// Elementwise kernels: the reference's extension ops taken one at a time
+// =============================================================================================
+
+__device__ __forceinline__ uint32_t nibble(uint32_t byte, int64_t i) {
+    return (i & 1) ? (byte & 0x0fu) : (byte >> 4);
+}
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T *x, int64_t i);
+template <>
+__device__ __forceinline__ float ldf<float>(const float *x, int64_t i) { return x[i]; }
+template <>
+__device__ __forceinline__ float ldf<uint16_t>(const uint16_t *x, int64_t i) { return bf2f(x[i]); }
+__device__ __forceinline__ void stf(float *x, int64_t i, float v) { x[i] = v; }
+__device__ __forceinline__ void stf(uint16_t *x, int64_t i, float v) { x[i] = (uint16_t)f2bf(v); }
+
+// x += alpha * (code * u + min); one thread per 8 elements
+template <typename T>
+__global__ __launch_bounds__(kWG) void quant_inv_kernel(int64_t d, int64_t q, const uint8_t *xq,
+                                                        const uint16_t *xmin,
+                                                        const uint16_t *xmax, T *x, float alpha) {
+    const int64_t i0 = ((int64_t)blockIdx.x * kWG + threadIdx.x) * kChunk;
+    if (i0 >= d) return;
+    const int n = (int)((d - i0) < kChunk ? (d - i0) : kChunk);
+    const bool vec = ((uintptr_t)(x + i0) & 15) == 0;
+    float v[8];
+    load8(x + i0, 0, n, vec, v);
+    int64_t b = i0 / q;
+    int64_t rem = i0 - b * q;
+    float mn = bf2f(xmin[b]), mx = bf2f(xmax[b]);
+    float u = (mx - mn) / 15.0f;
+#pragma unroll
+    for (int e = 0; e < kChunk; ++e) {
+        if (e < n) {
+            if (rem == q) {
+                rem = 0;
+                ++b;
+                mn = bf2f(xmin[b]);
+                mx = bf2f(xmax[b]);
+                u = (mx - mn) / 15.0f;
+            }
+            const uint32_t code = nibble(xq[(i0 + e) >> 1], i0 + e);
+            float deq = (float)code * u;
+            deq = deq + mn;
+            const float add = alpha * deq;
+            v[e] = v[e] + add;
+            ++rem;
+        }
+    }
+    store8(x + i0, 0, n, vec, v);
+}
+
+__device__ __forceinline__ uint32_t quant_code(float x, float mn, float u, bool ok) {
+    float v = (x - mn) / u;
+    v = floorf(v + 0.5f);
+    v = fmaxf(v, 0.0f);
+    v = fminf(v, 15.0f);
+    return ok ? (uint32_t)(int)v : 0u;
+}
+
+// xq = Q(x); one thread per 8 elements = 4 bytes of codes
+template <typename T>
+__global__ __launch_bounds__(kWG) void quant_kernel(int64_t d, int64_t q, uint8_t *xq,
+                                                    const uint16_t *xmin, const uint16_t *xmax,
+                                                    const T *x) {
+    const int64_t i0 = ((int64_t)blockIdx.x * kWG + threadIdx.x) * kChunk;
+    if (i0 >= d) return;
+    const int n = (int)((d - i0) < kChunk ? (d - i0) : kChunk);
+    const bool vec = ((uintptr_t)(x + i0) & 15) == 0;
+    float v[8];
+    load8(x + i0, 0, n, vec, v);
+    int64_t b = i0 / q;
+    int64_t rem = i0 - b * q;
+    float mn = bf2f(xmin[b]), mx = bf2f(xmax[b]);
+    float u = (mx - mn) / 15.0f;
+    bool ok = u != 0.0f && isfinite(u);
+    uint32_t codes[8];
+#pragma unroll
+    for (int e = 0; e < kChunk; ++e) {
+        codes[e] = 0;
+        if (e < n) {
+            if (rem == q) {
+                rem = 0;
+                ++b;
+                mn = bf2f(xmin[b]);
+                mx = bf2f(xmax[b]);
+                u = (mx - mn) / 15.0f;
+                ok = u != 0.0f && isfinite(u);
+            }
+            codes[e] = quant_code(v[e], mn, u, ok);
+            ++rem;
+        }
+    }
+    uint8_t *dst = xq + (i0 >> 1);
+    const int nbytes = (n + 1) >> 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (j < nbytes) dst[j] = (uint8_t)((codes[2 * j] << 4) | codes[2 * j + 1]);
+}
+
+// bf16 min / max per quantisation block.  per_wave != 0: each wave takes whole blocks in turn
+// (small q); else one workgroup per block.
+template <typename T>
+__global__ __launch_bounds__(kWG) void minmax_kernel(int64_t d, int64_t q, int64_t nblocks,
+                                                     const T *x, uint16_t *xmin, uint16_t *xmax,
+                                                     int per_wave) {
+    __shared__ float smn[kWaves], smx[kWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (per_wave) {
+        for (int64_t b = (int64_t)blockIdx.x * kWaves + wave; b < nblocks;
+             b += (int64_t)gridDim.x * kWaves) {
+            const int64_t lo = b * q, hi = (lo + q < d) ? lo + q : d;
+            float mn = INFINITY, mx = -INFINITY;
+            for (int64_t i = lo + lane; i < hi; i += kWave) {
+                const float v = ldf(x, i);
+                mn = v < mn ? v : mn;
+                mx = v > mx ? v : mx;
+            }
+#pragma unroll
+            for (int s = 32; s > 0; s >>= 1) {
+                const float a = __shfl_xor(mn, s, kWave), c = __shfl_xor(mx, s, kWave);
+                mn = a < mn ? a : mn;
+                mx = c > mx ? c : mx;
+            }
+            if (lane == 0) {
+                xmin[b] = (uint16_t)f2bf(mn);
+                xmax[b] = (uint16_t)f2bf(mx);
+            }
+        }
+    } else {
+        for (int64_t b = blockIdx.x; b < nblocks; b += gridDim.x) {
+            const int64_t lo = b * q, hi = (lo + q < d) ? lo + q : d;
+            float mn = INFINITY, mx = -INFINITY;
+            for (int64_t i = lo + tid; i < hi; i += kWG) {
+                const float v = ldf(x, i);
+                mn = v < mn ? v : mn;
+                mx = v > mx ? v : mx;
+            }
+#pragma unroll
+            for (int s = 32; s > 0; s >>= 1) {
+                const float a = __shfl_xor(mn, s, kWave), c = __shfl_xor(mx, s, kWave);
+                mn = a < mn ? a : mn;
+                mx = c > mx ? c : mx;
+            }
+            if (lane == 0) {
+                smn[wave] = mn;
+                smx[wave] = mx;
+            }
+            __syncthreads();
+            if (tid == 0) {
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w) {
+                    mn = smn[w] < mn ? smn[w] : mn;
+                    mx = smx[w] > mx ? smx[w] : mx;
+                }
+                xmin[b] = (uint16_t)f2bf(mn);
+                xmax[b] = (uint16_t)f2bf(mx);
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWG) void copy_values_kernel(int64_t k, int64_t dbs, int64_t kbs,
+                                                          const int16_t *idx, const void *inp,
+                                                          void *out, int direction) {
+    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (j >= k) return;
+    const int64_t pos = (j / kbs) * dbs + idx[j];
+    if (direction == 1)
+        ((uint16_t *)out)[j] = (uint16_t)f2bf(ldf((const T *)inp, pos));
+    else
+        stf((T *)out, pos, bf2f(((const uint16_t *)inp)[j]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWG) void zerorize_kernel(T *vec, const int16_t *idx, int64_t k,
+                                                       int64_t dbs, int64_t kbs) {
+    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (j >= k) return;
+    vec[(j / kbs) * dbs + idx[j]] = (T)0;
+}
+
+// p = rne(p * decay) (optional); p = rne(p + neg_lr * u); one thread per 8 elements
+template <typename T>
+__global__ __launch_bounds__(kWG) void param_update_kernel(int64_t d, T *p, const T *u,
+                                                           float neg_lr, int apply_decay,
+                                                           float decay) {
+    const int64_t i0 = ((int64_t)blockIdx.x * kWG + threadIdx.x) * kChunk;
+    if (i0 >= d) return;
+    const int n = (int)((d - i0) < kChunk ? (d - i0) : kChunk);
+    const bool vec = (((uintptr_t)(p + i0) | (uintptr_t)(u + i0)) & 15) == 0;
+    float pv[8], uv[8];
+    load8(p + i0, 0, n, vec, pv);
+    load8(u + i0, 0, n, vec, uv);
+#pragma unroll
+    for (int e = 0; e < kChunk; ++e) {
+        float x = pv[e];
+        if (apply_decay) {
+            x = x * decay;
+            if (sizeof(T) == 2) x = bf2f(f2bf(x));
+        }
+        const float prod = neg_lr * uv[e];
+        pv[e] = x + prod;
+    }
+    store8(p + i0, 0, n, vec, pv);
+}
+
+// =============================================================================================
+// Block kernels: one workgroup per top-k block, the block held in registers
+// =============================================================================================
+
+// LDS map shared by the block kernels (byte offsets from the start of dynamic LDS)
+struct LdsMap {
+    int off_sel_idx;  // uint16[kb_max]
+    int off_sel_val;  // uint16[kb_max]
+    int off_slot;     // slot_t[slot_cells]
+    int off_union;    // histogram (32 KiB) during selection, then z1 | z2 | coord
+    int slot_cells;   // multiple of 8, >= longest block
+    int z_cap;        // rows of z1 / z2 / coord
+    int sub_len;      // coordinates handled per window pass
+    int total;        // bytes
+};
+constexpr int kMiscBytes = 64;  // sh[8] words + counter at the very start
+constexpr int kHistBytes = 256 * kHistCopies * 4;
+
+struct WindowWeights {
+    float w1[kMaxWindow];
+    float w2[kMaxWindow];
+    float s1, s2, eps;
+    int rows;
+};
+
+// ---- standalone top-k (+ gather + zero) ---------------------------------------------------------
+
+template <class R>
+__global__ __launch_bounds__(kWG) void block_topk_kernel(int64_t d, int dbs, int k_many,
+                                                         int k_few, typename R::elem_t *x,
+                                                         int16_t *I_row, uint16_t *V_row,
+                                                         int zero_selected, LdsMap L) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
+    uint16_t *sel_idx = reinterpret_cast<uint16_t *>(lds + L.off_sel_idx);
+    uint16_t *sel_val = reinterpret_cast<uint16_t *>(lds + L.off_sel_val);
+    uint32_t *hist = reinterpret_cast<uint32_t *>(lds + L.off_union);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t b = blockIdx.x;
+    const int64_t n_full = d / dbs;
+    const int64_t e0 = b * dbs;
+    const int n = (int)((d - e0) < dbs ? (d - e0) : dbs);
+    const int kb = b < n_full ? k_many : k_few;
+    const int64_t col0 = b * k_many;
+    typename R::elem_t *xb = x + e0;
+    const bool vec = ((uintptr_t)xb & 15) == 0;
+
+    R r;
+    load_block(r, xb, n, vec, wave, lane);
+    uint32_t T;
+    int take_eq;
+    select_threshold(r, kb, hist, sh, T, take_eq);
+    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
+    for (int j = tid; j < kb; j += kWG) {
+        const int idx = sel_idx[j];
+        I_row[col0 + j] = (int16_t)idx;
+        if (V_row) V_row[col0 + j] = sel_val[j];
+        if (zero_selected) xb[idx] = (typename R::elem_t)0;
+    }
+}
+
+// ---- standalone Adam direction from the window ---------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(kWG) void window_update_kernel(int64_t d, int dbs, int kbs,
+                                                            int64_t k, const int16_t *I,
+                                                            const uint16_t *V, T *out,
+                                                            WindowWeights W, LdsMap L) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
+    uint32_t *counter = sh + 8;
+    uint16_t *slot = reinterpret_cast<uint16_t *>(lds + L.off_slot);
+    float *z1 = reinterpret_cast<float *>(lds + L.off_union);
+    float *z2 = z1 + L.z_cap;
+    uint16_t *coord = reinterpret_cast<uint16_t *>(z2 + L.z_cap);
+    const int tid = threadIdx.x;
+    const int64_t b = blockIdx.x;
+    const int64_t e0 = b * dbs;
+    const int n = (int)((d - e0) < dbs ? (d - e0) : dbs);
+    const int64_t col0 = b * kbs;
+    const int kb = (int)((k - col0) < kbs ? (k - col0) : kbs);
+
+    WindowView wv;
+    wv.I = I + col0;
+    wv.V = V + col0;
+    wv.k = k;
+    wv.rows = W.rows;
+    wv.cur_row = -1;
+    wv.cur_idx = nullptr;
+    wv.cur_val = nullptr;
+    wv.w1 = W.w1;
+    wv.w2 = W.w2;
+    for (int i = tid; i < L.slot_cells; i += kWG) slot[i] = 0;
+    for (int lo = 0; lo < n; lo += L.sub_len) {
+        const int hi = lo + L.sub_len < n ? lo + L.sub_len : n;
+        window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, L.z_cap);
+        const int cnt = (int)(*counter < (uint32_t)L.z_cap ? *counter : (uint32_t)L.z_cap);
+        for (int s = tid; s < cnt; s += kWG)
+            stf(out, e0 + coord[s], adam_direction(z1[s], z2[s], W.s1, W.s2, W.eps));
+        __syncthreads();
+    }
+}
+
+// ---- the fused step -----------------------------------------------------------------------------------
+
+struct TensorDesc {
+    void *p;
+    const void *g;
+    uint8_t *err;
+    uint16_t *mn;
+    uint16_t *mx;
+    int16_t *I;
+    uint16_t *V;
+    int64_t d;
+    int64_t k;
+    int32_t row;
+    int32_t k_many;
+    int32_t k_few;
+    int32_t first_block;  // first workgroup of this tensor inside the launch
+    float neg_lr;
+    float decay;
+    int32_t apply_decay;
+    int32_t pad;
+};
+constexpr int kTensorsPerLaunch = 24;
+
+struct FusedParams {
+    TensorDesc t[kTensorsPerLaunch];
+    WindowWeights W;
+    LdsMap L;
+    int32_t n_tensors;
+    int32_t d_block_size;
+    int32_t q_shift;  // log2(quant_block_size)
+    int32_t pad;
+};
+
+template <class R>
+struct RawChunk;
+template <int C>
+struct RawChunk<RegsBF16<C>> {
+    uint4 q;
+    __device__ __forceinline__ void load(const uint16_t *base, int off, int n) {
+        if (off + kChunk <= n) {
+            q = *reinterpret_cast<const uint4 *>(base + off);
+        } else {
+            uint32_t r[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (off + i < n) r[i >> 1] |= (uint32_t)base[off + i] << (16 * (i & 1));
+            q = make_uint4(r[0], r[1], r[2], r[3]);
+        }
+    }
+    __device__ __forceinline__ void to_float(float (&v)[8]) const {
+        const uint32_t r[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(r[i] << 16);
+            v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+        }
+    }
+};
+template <int C>
+struct RawChunk<RegsF32<C>> {
+    float v_[8];
+    __device__ __forceinline__ void load(const float *base, int off, int n) {
+        load8(base, off, n, true, v_);
+    }
+    __device__ __forceinline__ void to_float(float (&v)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = v_[i];
+    }
+};
+
+template <class R>
+__global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
+    typedef typename R::elem_t elem_t;
+    typedef typename R::slot_t slot_t;
+    constexpr int C = R::kC;
+    extern __shared__ __align__(16) unsigned char lds[];
+    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
+    uint32_t *counter = sh + 8;
+    uint16_t *sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
+    uint16_t *sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
+    slot_t *slot = reinterpret_cast<slot_t *>(lds + P.L.off_slot);
+    uint32_t *hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
+    float *z1 = reinterpret_cast<float *>(lds + P.L.off_union);
+    float *z2 = z1 + P.L.z_cap;
+    uint16_t *coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // which tensor, which block
+    int ti = 0;
+    for (int i = 1; i < P.n_tensors; ++i)
+        if ((int)blockIdx.x >= P.t[i].first_block) ti = i;
+    const TensorDesc &D = P.t[ti];
+    const int64_t b = (int)blockIdx.x - D.first_block;
+    const int64_t d = D.d;
+    const int dbs = (int)(d < P.d_block_size ? d : P.d_block_size);
+    const int64_t n_full = d / dbs;
+    const int64_t e0 = b * dbs;
+    const int n = (int)((d - e0) < dbs ? (d - e0) : dbs);
+    const int kb = b < n_full ? D.k_many : D.k_few;
+    const int64_t col0 = b * D.k_many;
+    const elem_t *g = reinterpret_cast<const elem_t *>(D.g) + e0;
+    elem_t *p = reinterpret_cast<elem_t *>(D.p) + e0;
+    uint8_t *err = D.err + (e0 >> 1);
+    const int q_shift = P.q_shift;
+    const int ql = 1 << (q_shift - 3);  // lanes per quantisation block
+
+    // ---- parameters: issued first, consumed last
+    RawChunk<R> praw[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n);
+
+    // ---- a = g + Qinv(e), rounded to the element type (MA:190)
+    R r;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int off = chunk_off<C>(wave, c, lane);
+        float v[8];
+        load8(g, off, n, true, v);
+        uint32_t cw = 0;
+        float mn = 0.0f, mx = 0.0f;
+        if (off < n) {
+            if (off + kChunk <= n) {
+                cw = *reinterpret_cast<const uint32_t *>(err + (off >> 1));
+            } else {
+                const int nbytes = (n - off + 1) >> 1;
+                for (int j = 0; j < nbytes; ++j) cw |= (uint32_t)err[(off >> 1) + j] << (8 * j);
+            }
+            const int64_t qb = (e0 + off) >> q_shift;
+            mn = bf2f(D.mn[qb]);
+            mx = bf2f(D.mx[qb]);
+        }
+        const float u = (mx - mn) / 15.0f;
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            const uint32_t code = (cw >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+            float deq = (float)code * u;
+            deq = deq + mn;
+            v[e] = v[e] + deq;
+        }
+        if (off + kChunk > n) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e)
+                if (off + e >= n) v[e] = 0.0f;
+        }
+        r.set_chunk(c, v);
+    }
+
+    // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214)
+    uint32_t T;
+    int take_eq;
+    select_threshold(r, kb, hist, sh, T, take_eq);
+    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
+    {
+        int16_t *Irow = D.I + (int64_t)D.row * D.k + col0;
+        uint16_t *Vrow = D.V + (int64_t)D.row * D.k + col0;
+        for (int j = tid; j < kb; j += kWG) {
+            Irow[j] = (int16_t)sel_idx[j];
+            Vrow[j] = sel_val[j];
+        }
+    }
+
+    // ---- residual statistics (MA:217-228) and 4-bit codes (MA:231)
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int off = chunk_off<C>(wave, c, lane);
+        float x[8];
+        float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            x[e] = r.val(c, e);
+            if (off + e < n) {
+                mn = x[e] < mn ? x[e] : mn;
+                mx = x[e] > mx ? x[e] : mx;
+            }
+        }
+        for (int s = 1; s < ql; s <<= 1) {
+            const float a = __shfl_xor(mn, s, kWave), c2 = __shfl_xor(mx, s, kWave);
+            mn = a < mn ? a : mn;
+            mx = c2 > mx ? c2 : mx;
+        }
+        const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
+        if (off < n) {
+            if ((lane & (ql - 1)) == 0) {
+                const int64_t qb = (e0 + off) >> q_shift;
+                D.mn[qb] = (uint16_t)mnb;
+                D.mx[qb] = (uint16_t)mxb;
+            }
+            const float mnf = bf2f(mnb), mxf = bf2f(mxb);
+            const float u = (mxf - mnf) / 15.0f;
+            const bool ok = u != 0.0f && isfinite(u);
+            uint32_t cw = 0;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const uint32_t code = (off + e < n) ? quant_code(x[e], mnf, u, ok) : 0u;
+                cw |= code << (8 * (e >> 1) + ((e & 1) ? 0 : 4));
+            }
+            if (off + kChunk <= n) {
+                *reinterpret_cast<uint32_t *>(err + (off >> 1)) = cw;
+            } else {
+                const int nbytes = (n - off + 1) >> 1;
+                for (int j = 0; j < nbytes; ++j) err[(off >> 1) + j] = (uint8_t)(cw >> (8 * j));
+            }
+        }
+    }
+
+    // ---- Adam direction from the window (MA:277-291); the slot cells end up holding the
+    //      update's bits, 0 where no window row names the coordinate
+    __syncthreads();  // the histogram's LDS is reused below
+    for (int i = tid; i < P.L.slot_cells; i += kWG) slot[i] = 0;
+    WindowView wv;
+    wv.I = D.I + col0;
+    wv.V = D.V + col0;
+    wv.k = D.k;
+    wv.rows = P.W.rows;
+    wv.cur_row = D.row;
+    wv.cur_idx = sel_idx;
+    wv.cur_val = sel_val;
+    wv.w1 = P.W.w1;
+    wv.w2 = P.W.w2;
+    for (int lo = 0; lo < n; lo += P.L.sub_len) {
+        const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+        window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
+        const int cnt = (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
+        for (int s = tid; s < cnt; s += kWG) {
+            const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
+            slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+        }
+        __syncthreads();
+    }
+
+    // ---- p = p * (1 - lr*wd) (MA:234-235); p += -lr * u (MA:304)
+    const float neg_lr = D.neg_lr, decay = D.decay;
+    const bool apply_decay = D.apply_decay != 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int off = chunk_off<C>(wave, c, lane);
+        if (off < n) {
+            float pv[8], uv[8];
+            praw[c].to_float(pv);
+            if (R::kBF16) {
+                const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
+                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uv[2 * i] = __uint_as_float(w[i] << 16);
+                    uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                }
+            } else {
+                const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
+                const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
+                uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
+                uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
+                uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
+                uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
+            }
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                float x = pv[e];
+                if (apply_decay) {
+                    x = x * decay;
+                    if (R::kBF16) x = bf2f(f2bf(x));
+                }
+                const float prod = neg_lr * uv[e];
+                pv[e] = x + prod;
+            }
+            store8(p, off, n, true, pv);
+        }
+    }
+}
+
+// =============================================================================================
+// Host side
+// =============================================================================================
+
+static inline int align16(int x) { return (x + 15) & ~15; }
+
+// LDS plan for a block kernel: longest block `dbs_max`, most entries per block row `kb_max`,
+// window length m, bytes per slot cell.
+static LdsMap plan_lds(int dbs_max, int kb_max, int m, int slot_bytes) {
+    LdsMap L;
+    L.off_sel_idx = kMiscBytes;
+    L.off_sel_val = L.off_sel_idx + align16(kb_max * 2);
+    L.off_slot = L.off_sel_val + align16(kb_max * 2);
+    L.slot_cells = (dbs_max + 7) & ~7;
+    L.off_union = L.off_slot + align16(L.slot_cells * slot_bytes);
+    const int64_t entries = (int64_t)m * kb_max;
+    if (entries <= 4096) {
+        L.sub_len = L.slot_cells;
+        L.z_cap = (int)(entries < 8 ? 8 : entries);
+    } else {
+        L.sub_len = 4096;
+        L.z_cap = 4096;
+    }
+    const int zbytes = L.z_cap * 10;
+    L.total = L.off_union + align16(zbytes > kHistBytes ? zbytes : kHistBytes);
+    return L;
+}
+
+static void window_weights(int64_t t, int m, double beta1, double beta2, double eps,
+                           WindowWeights *W) {
+    memset(W, 0, sizeof *W);
+    for (int i = 0; i < m; ++i) {
+        const int64_t age = ((t - 1 - i) % m + m) % m;
+        W->w1[i] = (float)pow(beta1, (double)age);
+        W->w2[i] = (float)pow(beta2, (double)age);
+    }
+    W->s1 = (float)((1.0 - beta1) / (1.0 - pow(beta1, (double)t)));
+    W->s2 = (float)((1.0 - beta2) / (1.0 - pow(beta2, (double)t)));
+    W->eps = (float)eps;
+    W->rows = (int)(t < m ? t : m);
+}
+
+static inline int launch_status() { return (int)hipGetLastError(); }
+
+static inline unsigned grid_for(int64_t work_items) {
+    return (unsigned)((work_items + kWG - 1) / kWG);
+}
+
+template <class K>
+static int allow_big_lds(K kernel, int bytes) {
+    if (bytes <= 64 * 1024) return 0;
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+constexpr int kLdsLimit = 160 * 1024;
+
+// chunks per thread that cover a block of `dbs` elements; 0 if none does
+static int chunks_for(int64_t dbs) {
+    if (dbs <= 2048 * 2) return 2;
+    if (dbs <= 2048 * 5) return 5;
+    if (dbs <= 2048 * 10) return 10;
+    if (dbs <= 2048 * 16) return 16;
+    return 0;
+}
+
+template <template <int> class RT>
+static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64_t d, int dbs,
+                       int k_many, int k_few, void *x, int16_t *I_row, uint16_t *V_row,
+                       int zero_selected, const LdsMap &L) {
+#define MA_TOPK_CASE(CC)                                                                     \
+    case CC: {                                                                               \
+        int rc = allow_big_lds(block_topk_kernel<RT<CC>>, lds_bytes);                        \
+        if (rc) return rc;                                                                   \
+        block_topk_kernel<RT<CC>><<<grid, kWG, lds_bytes, s>>>(                              \
+            d, dbs, k_many, k_few, (typename RT<CC>::elem_t *)x, I_row, V_row, zero_selected, \
+            L);                                                                              \
+        return launch_status();                                                              \
+    }
+    switch (C) {
+        MA_TOPK_CASE(2)
+        MA_TOPK_CASE(5)
+        MA_TOPK_CASE(10)
+        MA_TOPK_CASE(16)
+    }
+#undef MA_TOPK_CASE
+    return MA_ERR_BLOCK_SIZE;
+}
+
+template <template <int> class RT>
+static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+#define MA_FUSED_CASE(CC)                                                     \
+    case CC: {                                                                \
+        int rc = allow_big_lds(fused_step_kernel<RT<CC>>, lds_bytes);         \
+        if (rc) return rc;                                                    \
+        fused_step_kernel<RT<CC>><<<grid, kWG, lds_bytes, s>>>(P);            \
+        return launch_status();                                               \
+    }
+    switch (C) {
+        MA_FUSED_CASE(2)
+        MA_FUSED_CASE(5)
+        MA_FUSED_CASE(10)
+        MA_FUSED_CASE(16)
+    }
+#undef MA_FUSED_CASE
+    return MA_ERR_BLOCK_SIZE;
+}
+
+// geometry of one tensor, micro_adam.py:77-82
+struct Geometry {
+    int64_t dbs, n_full, tail, k_many, k_few, k;
+};
+static Geometry geometry(int64_t d, int64_t d_block_size, double k_init) {
+    Geometry g;
+    g.dbs = d < d_block_size ? d : d_block_size;
+    g.n_full = d / g.dbs;
+    g.tail = d - g.n_full * g.dbs;
+    g.k_many = (int64_t)ceil((double)g.dbs * k_init);
+    g.k_few = (int64_t)ceil((double)g.tail * k_init);
+    g.k = g.n_full * g.k_many + g.k_few;
+    return g;
+}
+
+static int fused_check(const ma_tensor *t, const ma_hyper *h) {
+    if (!t || !h) return MA_ERR_ARG;
+    if (!t->p || !t->g || !t->error || !t->min_vals || !t->max_vals || !t->I || !t->V)
+        return MA_ERR_ARG;
+    if (t->d <= 0 || h->t < 1 || h->m < 1 || (h->dtype != MA_F32 && h->dtype != MA_BF16))
+        return MA_ERR_ARG;
+    if (h->m > MA_MAX_WINDOW) return MA_ERR_WINDOW;
+    if (h->d_block_size < 1 || h->quant_block_size < 1) return MA_ERR_ARG;
+    if (!(h->k_init > 0.0 && h->k_init <= 1.0)) return MA_ERR_ARG;
+    if (t->index < 0 || t->index >= h->m) return MA_ERR_ARG;
+    const Geometry g = geometry(t->d, h->d_block_size, h->k_init);
+    if (g.dbs > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    if (g.k != t->k) return MA_ERR_GEOMETRY;
+    const int64_t q = h->quant_block_size;
+    if (q < 8 || q > 512 || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
+    if (t->d < q) return MA_ERR_NOT_FUSABLE;
+    const bool single = t->d <= h->d_block_size;
+    if (!single && (g.dbs % q != 0 || g.dbs % 8 != 0)) return MA_ERR_NOT_FUSABLE;
+    if ((((uintptr_t)t->p | (uintptr_t)t->g) & 15) != 0 || ((uintptr_t)t->error & 3) != 0)
+        return MA_ERR_NOT_FUSABLE;
+    return 0;
+}
+
+}  // namespace ma
+
+using namespace ma;
+
+extern "C" {
+
+const char *ma_error_string(int code) {
+    switch (code) {
+        case 0: return "ok";
+        case MA_ERR_ARG: return "bad argument (null pointer, size, dtype or direction)";
+        case MA_ERR_BLOCK_SIZE: return "top-k block longer than 32768 elements";
+        case MA_ERR_WINDOW: return "window length m exceeds MA_MAX_WINDOW";
+        case MA_ERR_GEOMETRY: return "k / k_block_size inconsistent with d and d_block_size";
+        case MA_ERR_NOT_FUSABLE: return "tensor does not meet the fused step's layout conditions";
+        case MA_ERR_LDS: return "launch would need more than 160 KB of LDS";
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+int ma_get_sm_count(void) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        return -1;
+    return n;
+}
+
+int ma_get_max_floats_for_shared_memory_per_thread_block(void) {
+    return kLdsLimit / 4;  // gfx950: 160 KB of LDS per workgroup
+}
+
+#define MA_DISPATCH_DTYPE(dtype, CALL_F32, CALL_BF16) \
+    if ((dtype) == MA_F32) { CALL_F32; }              \
+    else if ((dtype) == MA_BF16) { CALL_BF16; }       \
+    else return MA_ERR_ARG;
+
+int ma_copy_values(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
+                   const int16_t *indices, const void *inp, void *out, int direction, int dtype,
+                   void *stream) {
+    if (!indices || !inp || !out || d <= 0 || k < 0 || d_block_size <= 0 || k_block_size <= 0)
+        return MA_ERR_ARG;
+    if (direction != 0 && direction != 1) return MA_ERR_ARG;
+    if (d_block_size > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    // every j must land inside d: the last block row may not reach past the tensor
+    if (((k + k_block_size - 1) / k_block_size - 1) * d_block_size >= d && k > 0)
+        return MA_ERR_GEOMETRY;
+    if (k == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    MA_DISPATCH_DTYPE(dtype,
+        (copy_values_kernel<float><<<grid_for(k), kWG, 0, s>>>(k, d_block_size, k_block_size,
+                                                                indices, inp, out, direction)),
+        (copy_values_kernel<uint16_t><<<grid_for(k), kWG, 0, s>>>(k, d_block_size, k_block_size,
+                                                                   indices, inp, out, direction)))
+    return launch_status();
+}
+
+int ma_zerorize_block_components(void *vector, const int16_t *indices, int64_t d, int64_t k,
+                                 int64_t d_block_size, int64_t k_block_size, int dtype,
+                                 void *stream) {
+    if (!vector || !indices || d <= 0 || k < 0 || d_block_size <= 0 || k_block_size <= 0)
+        return MA_ERR_ARG;
+    if (d_block_size > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    if (k > 0 && ((k + k_block_size - 1) / k_block_size - 1) * d_block_size >= d)
+        return MA_ERR_GEOMETRY;
+    if (k == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    MA_DISPATCH_DTYPE(dtype,
+        (zerorize_kernel<float><<<grid_for(k), kWG, 0, s>>>((float *)vector, indices, k,
+                                                            d_block_size, k_block_size)),
+        (zerorize_kernel<uint16_t><<<grid_for(k), kWG, 0, s>>>((uint16_t *)vector, indices, k,
+                                                               d_block_size, k_block_size)))
+    return launch_status();
+}
+
+int ma_asymm_block_quant(int64_t d, int64_t q, uint8_t *xq, const uint16_t *xmin,
+                         const uint16_t *xmax, const void *x, int dtype, void *stream) {
+    if (!xq || !xmin || !xmax || !x || d <= 0 || q <= 0) return MA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
+    MA_DISPATCH_DTYPE(dtype,
+        (quant_kernel<float><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (const float *)x)),
+        (quant_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (const uint16_t *)x)))
+    return launch_status();
+}
+
+int ma_asymm_block_quant_inv(int64_t d, int64_t q, const uint8_t *xq, const uint16_t *xmin,
+                             const uint16_t *xmax, void *x, float alpha, int dtype,
+                             void *stream) {
+    if (!xq || !xmin || !xmax || !x || d <= 0 || q <= 0) return MA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
+    MA_DISPATCH_DTYPE(dtype,
+        (quant_inv_kernel<float><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (float *)x, alpha)),
+        (quant_inv_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (uint16_t *)x,
+                                                         alpha)))
+    return launch_status();
+}
+
+int ma_block_minmax(int64_t d, int64_t q, const void *x, uint16_t *xmin, uint16_t *xmax,
+                    int dtype, void *stream) {
+    if (!x || !xmin || !xmax || d <= 0 || q <= 0) return MA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t nblocks = (d + q - 1) / q;
+    const int per_wave = q <= 1024;
+    int64_t wgs = per_wave ? (nblocks + kWaves - 1) / kWaves : nblocks;
+    if (wgs > 65536 * 16) wgs = 65536 * 16;
+    const unsigned grid = (unsigned)wgs;
+    MA_DISPATCH_DTYPE(dtype,
+        (minmax_kernel<float><<<grid, kWG, 0, s>>>(d, q, nblocks, (const float *)x, xmin, xmax,
+                                                   per_wave)),
+        (minmax_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, nblocks, (const uint16_t *)x, xmin,
+                                                      xmax, per_wave)))
+    return launch_status();
+}
+
+int ma_param_update(int64_t d, void *p, const void *u, float neg_lr, int apply_decay, float decay,
+                    int dtype, void *stream) {
+    if (!p || !u || d <= 0) return MA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
+    MA_DISPATCH_DTYPE(dtype,
+        (param_update_kernel<float><<<grid, kWG, 0, s>>>(d, (float *)p, (const float *)u, neg_lr,
+                                                         apply_decay, decay)),
+        (param_update_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, (uint16_t *)p,
+                                                            (const uint16_t *)u, neg_lr,
+                                                            apply_decay, decay)))
+    return launch_status();
+}
+
+int ma_block_topk(int64_t d, int64_t d_block_size, int64_t k_many, int64_t k_few, void *x,
+                  int16_t *I_row, uint16_t *V_row, int zero_selected, int dtype, void *stream) {
+    if (!x || !I_row || d <= 0 || d_block_size <= 0 || d_block_size > d) return MA_ERR_ARG;
+    if (dtype != MA_F32 && dtype != MA_BF16) return MA_ERR_ARG;
+    if (d_block_size > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    const int64_t n_full = d / d_block_size, tail = d - n_full * d_block_size;
+    if (k_many < 1 || k_many > d_block_size || k_few < 0 || k_few > tail || (tail > 0) != (k_few > 0))
+        return MA_ERR_GEOMETRY;
+    const int C = chunks_for(d_block_size);
+    if (!C) return MA_ERR_BLOCK_SIZE;
+    const LdsMap L = plan_lds((int)d_block_size, (int)k_many, 1, 2);
+    if (L.total > kLdsLimit) return MA_ERR_LDS;
+    const unsigned grid = (unsigned)(n_full + (tail > 0 ? 1 : 0));
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == MA_F32)
+        return launch_topk<RegsF32>(C, grid, L.total, s, d, (int)d_block_size, (int)k_many,
+                                    (int)k_few, x, I_row, V_row, zero_selected, L);
+    return launch_topk<RegsBF16>(C, grid, L.total, s, d, (int)d_block_size, (int)k_many,
+                                 (int)k_few, x, I_row, V_row, zero_selected, L);
+}
+
+int ma_compute_microadam_update(int blocks, int threads, int carveout, int64_t t, double beta1,
+                                double beta2, double eps, int64_t d_block_size,
+                                int64_t k_block_size, int64_t d, int64_t m, int64_t k,
+                                const int16_t *indices, const uint16_t *values, void *out,
+                                int dtype, void *stream) {
+    (void)blocks; (void)threads; (void)carveout;
+    if (!indices || !values || !out || d <= 0 || k <= 0 || t < 1 || m < 1) return MA_ERR_ARG;
+    if (d_block_size <= 0 || k_block_size <= 0 || k_block_size > d_block_size) return MA_ERR_ARG;
+    if (dtype != MA_F32 && dtype != MA_BF16) return MA_ERR_ARG;
+    if (m > MA_MAX_WINDOW) return MA_ERR_WINDOW;
+    if (d_block_size > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    const int64_t nblocks = (k + k_block_size - 1) / k_block_size;
+    // every block row must start inside the tensor
+    if ((nblocks - 1) * d_block_size >= d) return MA_ERR_GEOMETRY;
+    WindowWeights W;
+    window_weights(t, (int)m, beta1, beta2, eps, &W);
+    const LdsMap L = plan_lds((int)d_block_size, (int)k_block_size, (int)m, 2);
+    if (L.total > kLdsLimit) return MA_ERR_LDS;
+    hipStream_t s = (hipStream_t)stream;
+    int rc;
+    if (dtype == MA_F32) {
+        if ((rc = allow_big_lds(window_update_kernel<float>, L.total))) return rc;
+        window_update_kernel<float><<<(unsigned)nblocks, kWG, L.total, s>>>(
+            d, (int)d_block_size, (int)k_block_size, k, indices, values, (float *)out, W, L);
+    } else {
+        if ((rc = allow_big_lds(window_update_kernel<uint16_t>, L.total))) return rc;
+        window_update_kernel<uint16_t><<<(unsigned)nblocks, kWG, L.total, s>>>(
+            d, (int)d_block_size, (int)k_block_size, k, indices, values, (uint16_t *)out, W, L);
+    }
+    return launch_status();
+}
+
+int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
+    return fused_check(tensor, hyper);
+}
+
+int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream) {
+    if (!tensors || !h || n_tensors < 0) return MA_ERR_ARG;
+    for (int i = 0; i < n_tensors; ++i) {
+        const int rc = fused_check(&tensors[i], h);
+        if (rc) return rc;
+    }
+    if (n_tensors == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    int q_shift = 0;
+    while ((1LL << q_shift) < h->quant_block_size) ++q_shift;
+    WindowWeights W;
+    window_weights(h->t, h->m, h->beta1, h->beta2, h->eps, &W);
+    const int slot_bytes = h->dtype == MA_BF16 ? 2 : 4;
+
+    // launches are formed per register-tile size so that small tensors do not run in the
+    // largest kernel; inside a class, tensors go kTensorsPerLaunch at a time by value
+    static const int classes[4] = {2, 5, 10, 16};
+    for (int ci = 0; ci < 4; ++ci) {
+        const int C = classes[ci];
+        FusedParams P;
+        int count = 0;
+        int64_t blocks = 0;
+        int dbs_max = 0, kb_max = 0;
+        auto flush = [&]() -> int {
+            if (count == 0) return 0;
+            P.n_tensors = count;
+            P.W = W;
+            P.L = plan_lds(dbs_max, kb_max, h->m, slot_bytes);
+            P.d_block_size = (int)(h->d_block_size > MA_MAX_D_BLOCK ? MA_MAX_D_BLOCK
+                                                                     : h->d_block_size);
+            P.q_shift = q_shift;
+            P.pad = 0;
+            if (P.L.total > kLdsLimit) return MA_ERR_LDS;
+            const int rc = h->dtype == MA_BF16
+                               ? launch_fused<RegsBF16>(C, (unsigned)blocks, P.L.total, s, P)
+                               : launch_fused<RegsF32>(C, (unsigned)blocks, P.L.total, s, P);
+            count = 0;
+            blocks = 0;
+            dbs_max = kb_max = 0;
+            return rc;
+        };
+        for (int i = 0; i < n_tensors; ++i) {
+            const ma_tensor &t = tensors[i];
+            const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
+            if (chunks_for(g.dbs) != C) continue;
+            const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
+            if (count == kTensorsPerLaunch || blocks + nb > 0x7fffffff) {
+                const int rc = flush();
+                if (rc) return rc;
+            }
+            TensorDesc &D = P.t[count];
+            D.p = t.p;
+            D.g = t.g;
+            D.err = t.error;
+            D.mn = t.min_vals;
+            D.mx = t.max_vals;
+            D.I = t.I;
+            D.V = t.V;
+            D.d = t.d;
+            D.k = t.k;
+            D.row = t.index;
+            D.k_many = (int32_t)g.k_many;
+            D.k_few = (int32_t)g.k_few;
+            D.first_block = (int32_t)blocks;
+            D.neg_lr = (float)(-t.lr);
+            D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
+            D.decay = (float)(1.0 - t.lr * t.weight_decay);
+            D.pad = 0;
+            blocks += nb;
+            if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
+            if (g.k_many > kb_max) kb_max = (int)g.k_many;
+            ++count;
+        }
+        const int rc = flush();
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -292,7 +292,8 @@ void ora_zerorize_block_components(void *vector, const int16_t *indices, int64_t
  *   out = rne( (z1 * s1) / (eps + sqrtf(z2 * s2)) ),
  *   s1 = (1-beta1)/(1-beta1^t), s2 = (1-beta2)/(1-beta2^t) (double -> fp32),
  *   w[age] = (float)pow(beta, age).
- * Coordinates no live row names are left untouched (the caller zeroed out). */
+ * Coordinates that no live row names with a non-zero value are left untouched (the caller
+ * zeroed out, micro_adam.py:276, so they read as a zero update either way). */
 void ora_compute_microadam_update(int64_t t, double beta1, double beta2, double eps,
                                   int64_t d_block_size, int64_t k_block_size, int64_t d,
                                   int64_t m, int64_t k, const int16_t *indices,
@@ -328,6 +329,9 @@ void ora_compute_microadam_update(int64_t t, double beta1, double beta2, double 
                 const uint16_t *vr = values + r * k;
                 for (int64_t j = j0; j < j1; ++j) {
                     int idx = ir[j];
+                    /* a +-0 value adds nothing and does not mark its coordinate (rows of a
+                     * fresh window are all (index 0, value 0)) */
+                    if ((vr[j] & 0x7fffu) == 0) continue;
                     float v = bf16_to_f32(vr[j]);
                     float a1 = w1[r] * v;
                     float vv = v * v;
