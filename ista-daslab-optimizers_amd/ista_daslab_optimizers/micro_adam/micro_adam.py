@@ -190,16 +190,45 @@ class MicroAdam(torch.optim.Optimizer):
         if p.dtype not in (torch.float32, torch.bfloat16):
             raise TypeError(f"MicroAdam takes float32 or bfloat16 parameters, got {p.dtype}")
 
-    @staticmethod
-    def _repair_state(st):
-        # Optimizer.load_state_dict casts floating-point state to the parameter's dtype and
-        # some frameworks re-type st['I'] (micro_adam.py:175-178); the kernels need the
-        # declared types back.  The casts are lossless: the values were bf16 / int16.
-        if st['I'].dtype != torch.int16:
-            st['I'] = st['I'].to(torch.int16)
-        for key in ('V', 'min_vals', 'max_vals'):
-            if st[key].dtype != torch.bfloat16:
-                st[key] = st[key].to(torch.bfloat16)
+    _STATE_DTYPES = (('I', torch.int16), ('V', torch.bfloat16), ('error', torch.uint8),
+                     ('min_vals', torch.bfloat16), ('max_vals', torch.bfloat16))
+
+    @classmethod
+    def _repair_state(cls, st):
+        # Frameworks that reload or re-type optimizer state cast every state tensor to the
+        # parameter's dtype (the reference repairs st['I'] for this reason,
+        # micro_adam.py:175-178); the kernels need the declared types back.
+        for key, dtype in cls._STATE_DTYPES:
+            if st[key].dtype != dtype:
+                st[key] = st[key].to(dtype)
+
+    # ------------------------------------------------------------------ checkpointing
+    def state_dict(self):
+        """As torch's, plus the global step counter, which the reference keeps as a plain
+        attribute (micro_adam.py:35) and therefore loses on resume: the ages of the window
+        rows and the bias corrections depend on it."""
+        sd = super().state_dict()
+        sd['steps'] = self.steps
+        return sd
+
+    def load_state_dict(self, state_dict):
+        """torch's load_state_dict casts all per-parameter tensors to the parameter's dtype,
+        which would destroy int16 indices under bf16 parameters; the typed tensors are taken
+        from the source dictionary again afterwards."""
+        super().load_state_dict(state_dict)
+        if 'steps' in state_dict:
+            self.steps = int(state_dict['steps'])
+        saved_ids = [pid for g in state_dict['param_groups'] for pid in g['params']]
+        params = [p for g in self.param_groups for p in g['params']]
+        for pid, p in zip(saved_ids, params):
+            saved = state_dict['state'].get(pid)
+            if saved is None:
+                continue
+            st = self.state[p]
+            for key, dtype in self._STATE_DTYPES:
+                if key in saved and torch.is_tensor(saved[key]) and saved[key].dtype == dtype:
+                    st[key] = saved[key].to(device=p.device, copy=True)
+        self._fused_cache = None
 
     def _fusable(self, p, st):
         if self.alpha != 0:

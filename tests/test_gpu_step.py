@@ -169,7 +169,7 @@ def test_state_layout_and_checkpoint_roundtrip():
     p2 = torch.nn.Parameter(p.detach().clone())
     opt2 = MicroAdam([p2], m=10, lr=1e-3, quant_block_size=64)
     opt2.load_state_dict(sd)
-    opt2.steps = opt.steps  # the reference does not persist the step counter (micro_adam.py:35)
+    assert opt2.steps == opt.steps  # the reference loses the counter on resume (micro_adam.py:35)
     g = torch.randn_like(p) * 1e-2
     p.grad, p2.grad = g.clone(), g.clone()
     opt.step()
@@ -178,6 +178,16 @@ def test_state_layout_and_checkpoint_roundtrip():
     assert torch.equal(p.data, p2.data)
     for key in ("I", "V", "error", "min_vals", "max_vals"):
         assert torch.equal(opt.state[p][key], opt2.state[p2][key]), key
+    # a framework that re-types the state (every tensor cast to the parameter's dtype) is
+    # repaired on the next step, as the reference does for st['I']
+    st2 = opt2.state[p2]
+    for key in ("I", "V", "error", "min_vals", "max_vals"):
+        st2[key] = st2[key].to(torch.float32)
+    p.grad, p2.grad = g.clone(), g.clone()
+    opt.step()
+    opt2.step()
+    assert st2["I"].dtype == torch.int16 and st2["error"].dtype == torch.uint8
+    assert torch.equal(p.data, p2.data)
 
 
 def test_cpu_parameter_is_rejected():
