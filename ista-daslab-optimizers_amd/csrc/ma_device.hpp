@@ -19,6 +19,29 @@ constexpr int kChunk = 8;        // elements per lane per chunk
 constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
 constexpr int kMaxWindow = 64;
 
+// ---- development aid ---------------------------------------------------------------------------
+// With MA_PHASE_TIMING (never defined in the shipped build) thread 0 of every workgroup adds
+// the cycles between marks into a caller-provided buffer; otherwise the timer is empty.
+#ifdef MA_PHASE_TIMING
+__device__ unsigned long long *g_phase_buf = nullptr;
+struct PhaseTimer {
+    unsigned long long t;
+    __device__ __forceinline__ void begin() { t = __builtin_readcyclecounter(); }
+    __device__ __forceinline__ void mark(int i) {
+        if (threadIdx.x == 0 && g_phase_buf) {
+            const unsigned long long now = __builtin_readcyclecounter();
+            atomicAdd(&g_phase_buf[i], now - t);
+            t = now;
+        }
+    }
+};
+#else
+struct PhaseTimer {
+    __device__ __forceinline__ void begin() {}
+    __device__ __forceinline__ void mark(int) {}
+};
+#endif
+
 // ---- scalar helpers -----------------------------------------------------------------------
 
 __device__ __forceinline__ float bf2f(uint32_t h) { return __uint_as_float(h << 16); }
@@ -42,13 +65,52 @@ __device__ __forceinline__ uint32_t mbcnt(uint64_t mask) {
                                      __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
+// Value of the DPP source lane, 0 where the pattern has no source or the lane is masked off.
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ uint32_t dpp_or0(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, BANK_MASK, false);
+}
+
+// Inclusive prefix sum over the 64 lanes, all in the VALU (no LDS round trips).
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        uint32_t t = __shfl_up(v, d, kWave);
-        if (lane >= d) v += t;
-    }
+    (void)lane;
+    v += dpp_or0<0x111>(v);             // row_shr:1
+    v += dpp_or0<0x112>(v);             // row_shr:2
+    v += dpp_or0<0x114, 0xF, 0xE>(v);   // row_shr:4, lanes 4..15 of each row
+    v += dpp_or0<0x118, 0xF, 0xC>(v);   // row_shr:8, lanes 8..15 of each row
+    v += dpp_or0<0x142, 0xA>(v);        // row_bcast:15 into rows 1 and 3
+    v += dpp_or0<0x143, 0xC>(v);        // row_bcast:31 into rows 2 and 3
     return v;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_perm(float v) {
+    return __int_as_float(
+        __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// min / max over aligned groups of `ql` lanes (a power of two), result in every lane
+__device__ __forceinline__ void group_minmax(float &mn, float &mx, int ql) {
+    if (ql >= 2) {
+        mn = __builtin_fminf(mn, dpp_perm<0xB1>(mn));  // quad_perm [1,0,3,2]
+        mx = __builtin_fmaxf(mx, dpp_perm<0xB1>(mx));
+    }
+    if (ql >= 4) {
+        mn = __builtin_fminf(mn, dpp_perm<0x4E>(mn));  // quad_perm [2,3,0,1]
+        mx = __builtin_fmaxf(mx, dpp_perm<0x4E>(mx));
+    }
+    if (ql >= 8) {
+        mn = __builtin_fminf(mn, dpp_perm<0x141>(mn));  // row_half_mirror
+        mx = __builtin_fmaxf(mx, dpp_perm<0x141>(mx));
+    }
+    if (ql >= 16) {
+        mn = __builtin_fminf(mn, dpp_perm<0x140>(mn));  // row_mirror
+        mx = __builtin_fmaxf(mx, dpp_perm<0x140>(mx));
+    }
+    for (int s = 16; s < ql; s <<= 1) {
+        mn = __builtin_fminf(mn, __shfl_xor(mn, s, kWave));
+        mx = __builtin_fmaxf(mx, __shfl_xor(mx, s, kWave));
+    }
 }
 
 // Inclusive scan over the 256 threads in thread order.  sh4 is 4 words of LDS.
@@ -195,16 +257,28 @@ __device__ __forceinline__ void load_block(R &r, const typename R::elem_t *base,
     }
 }
 
+// Keeps the compiler from carrying values derived from the block registers (unpacked keys,
+// widened floats) from one phase into the next: after this it only knows the registers.
+template <class R>
+__device__ __forceinline__ void launder(R &r) {
+#pragma unroll
+    for (int c = 0; c < R::kC; ++c) {
+#pragma unroll
+        for (int i = 0; i < (R::kBF16 ? 4 : 8); ++i) asm volatile("" : "+v"(r.w[c][i]));
+    }
+}
+
 // ---- threshold search: MSD radix select over the magnitude bits -----------------------------
 //
 // Finds the key T of the kb-th largest magnitude and how many entries equal to T belong to
 // the top kb (`take_eq` >= 1).  Each pass histograms one digit of the keys that still match
 // the prefix into `hist`, 32 replicated copies per bin so that every lane adds into its own
 // LDS bank whatever the data look like, then scans the bins from the top.
-//   hist: 256*32 words, sh: 8 words.  Ends with a barrier.
+//   hist: 257*32 words (bin 256 is a discard bin), sh: 8 words.  Ends with a barrier.
 template <class R>
-__device__ __forceinline__ void select_threshold(const R &r, int kb, uint32_t *hist, uint32_t *sh,
-                                                 uint32_t &T, int &take_eq) {
+__device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, uint32_t *sh,
+                                                 uint32_t &T, int &take_eq, PhaseTimer &pt,
+                                                 int pt0) {
     constexpr int kPasses = R::kBF16 ? 2 : 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t prefix = 0, pmask = 0;
@@ -217,17 +291,22 @@ __device__ __forceinline__ void select_threshold(const R &r, int kb, uint32_t *h
         const uint32_t dm = nb - 1;
         for (int i = tid; i < nb * kHistCopies / 4; i += kWG)
             reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+        launder(r);
         __syncthreads();
+        if (pass < 2) pt.mark(pt0 + 3 * pass);
 #pragma unroll
         for (int c = 0; c < R::kC; ++c) {
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                uint32_t key = r.key(c, e);
-                if ((key & pmask) == prefix)
-                    atomicAdd(&hist[(((key >> shift) & dm) << 5) + (lane & 31)], 1u);
+                const uint32_t key = r.key(c, e);
+                // keys off the prefix count into a spare bin: cheaper than branching
+                const uint32_t bin = (key & pmask) == prefix ? ((key >> shift) & dm) : 256u;
+                atomicAdd(&hist[(bin << 5) + (lane & 31)], 1u);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
+        if (pass < 2) pt.mark(pt0 + 3 * pass + 1);
         // thread tid owns bin nb-1-tid so that a forward scan walks the bins from the top
         const int bin = nb - 1 - tid;
         uint32_t cnt = 0;
@@ -245,6 +324,7 @@ __device__ __forceinline__ void select_threshold(const R &r, int kb, uint32_t *h
         prefix |= sh[4] << shift;
         pmask |= dm << shift;
         need = (int)sh[5];
+        if (pass < 2) pt.mark(pt0 + 3 * pass + 2);
     }
     __syncthreads();
     T = prefix;
@@ -259,7 +339,7 @@ __device__ __forceinline__ void select_threshold(const R &r, int kb, uint32_t *h
 template <class R>
 __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, int kb,
                                                  uint16_t *sel_idx, uint16_t *sel_val,
-                                                 uint32_t *sh) {
+                                                 uint32_t *sh, PhaseTimer &pt, int pt0) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t pre[R::kC];  // low 16: entries >= T before this lane's chunk; high 16: == T
     uint32_t run = 0;
@@ -273,14 +353,17 @@ __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, 
         }
         uint32_t incl = wave_incl_scan(cnt, lane);
         pre[c] = run + incl - cnt;
-        run += __shfl(incl, kWave - 1, kWave);
+        run += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
     if (lane == 0) sh[wave] = run;
+    launder(r);
     __syncthreads();
     uint32_t base = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
         if (w < wave) base += sh[w];
+    pt.mark(pt0);
 #pragma unroll
     for (int c = 0; c < R::kC; ++c) {
         uint32_t p = pre[c] + base;
@@ -302,8 +385,10 @@ __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, 
                 eq_before += is_eq ? 1u : 0u;
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+    pt.mark(pt0 + 1);
 }
 
 // ---- Adam statistics of one block from its window rows ---------------------------------------------
@@ -326,6 +411,42 @@ struct WindowView {
     const float *w1;    // beta1^age per row
     const float *w2;
 };
+
+// One window entry per thread: add (w1*v, w2*v*v) to the sums of coordinate idx, handing out
+// a fresh row of z1 / z2 / coord when the coordinate is seen for the first time.  Must be
+// called by every lane of the wave (inactive lanes pass active = false).
+template <typename slot_t>
+__device__ __forceinline__ void window_entry(int idx, uint32_t vb, bool active, float w1,
+                                             float w2, slot_t *slot, float *z1, float *z2,
+                                             uint16_t *coord, uint32_t *counter, int cap,
+                                             int lane) {
+    const float v = bf2f(vb);
+    const float a1 = w1 * v;
+    const float vv = v * v;
+    const float a2 = w2 * vv;
+    uint32_t s = active ? (uint32_t)slot[idx] : 1u;
+    const bool fresh = active && s == 0;
+    const uint64_t mask = __ballot(fresh);
+    if (mask != 0) {
+        const int leader = __ffsll((unsigned long long)mask) - 1;
+        uint32_t first = 0;
+        if (lane == leader) first = atomicAdd(counter, (uint32_t)__popcll(mask));
+        first = __shfl(first, leader, kWave);
+        if (fresh) {
+            s = first + mbcnt(mask) + 1;
+            if (s <= (uint32_t)cap) {  // always true for duplicate-free rows
+                slot[idx] = (slot_t)s;
+                coord[s - 1] = (uint16_t)idx;
+                z1[s - 1] = 0.0f + a1;
+                z2[s - 1] = 0.0f + a2;
+            }
+        }
+    }
+    if (active && !fresh) {
+        z1[s - 1] = z1[s - 1] + a1;
+        z2[s - 1] = z2[s - 1] + a2;
+    }
+}
 
 template <typename slot_t>
 __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, int lo, int hi,
@@ -355,35 +476,42 @@ __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, 
                 // window from naming coordinate 0 many times in one row
                 active = idx >= lo && idx < hi && (vb & 0x7fffu) != 0;
             }
-            const float v = bf2f(vb);
-            const float a1 = w1 * v;
-            const float vv = v * v;
-            const float a2 = w2 * vv;
-            uint32_t s = active ? (uint32_t)slot[idx] : 1u;
-            const bool fresh = active && s == 0;
-            const uint64_t mask = __ballot(fresh);
-            if (mask != 0) {
-                const int leader = __ffsll((unsigned long long)mask) - 1;
-                uint32_t first = 0;
-                if (lane == leader) first = atomicAdd(counter, (uint32_t)__popcll(mask));
-                first = __shfl(first, leader, kWave);
-                if (fresh) {
-                    s = first + mbcnt(mask) + 1;
-                    if (s <= (uint32_t)cap) {  // always true for duplicate-free rows
-                        slot[idx] = (slot_t)s;
-                        coord[s - 1] = (uint16_t)idx;
-                        z1[s - 1] = 0.0f + a1;
-                        z2[s - 1] = 0.0f + a2;
-                    }
-                }
-            }
-            if (active && !fresh) {
-                z1[s - 1] = z1[s - 1] + a1;
-                z2[s - 1] = z2[s - 1] + a2;
-            }
+            window_entry(idx, vb, active, w1, w2, slot, z1, z2, coord, counter, cap, lane);
         }
         __syncthreads();
     }
+}
+
+// ---- division by a value shared by many numerators ---------------------------------------------
+//
+// y / u, correctly rounded, with the refinement of 1/u paid once.  This is the fp32 division
+// expansion of the compiler (reciprocal, one Newton step, quotient, two fused residual
+// corrections) without its operand scaling and special-case fix-up, so it equals IEEE division
+// bit for bit whenever those would be no-ops: u normal and away from the ends of the exponent
+// range (`safe`), and the quotient neither overflowing nor denormal.  Callers keep |y| within a
+// few multiples of 16 u, and a quotient below 2^-30 is only ever compared with 1/2.
+struct Divisor {
+    float u, r;
+    bool safe;
+};
+
+__device__ __forceinline__ Divisor make_divisor(float u) {
+    Divisor d;
+    d.u = u;
+    const float r0 = __builtin_amdgcn_rcpf(u);
+    const float e = __builtin_fmaf(-u, r0, 1.0f);
+    d.r = __builtin_fmaf(e, r0, r0);
+    const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
+    d.safe = ex >= 32u && ex <= 222u;
+    return d;
+}
+
+__device__ __forceinline__ float div_shared(float y, const Divisor &d) {
+    const float q0 = y * d.r;
+    const float e1 = __builtin_fmaf(-d.u, q0, y);
+    const float q1 = __builtin_fmaf(e1, d.r, q0);
+    const float e2 = __builtin_fmaf(-d.u, q1, y);
+    return __builtin_fmaf(e2, d.r, q1);
 }
 
 __device__ __forceinline__ float adam_direction(float z1, float z2, float s1, float s2,

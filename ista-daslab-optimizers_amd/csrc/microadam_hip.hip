@@ -236,7 +236,7 @@ struct LdsMap {
     int total;        // bytes
 };
 constexpr int kMiscBytes = 64;  // sh[8] words + counter at the very start
-constexpr int kHistBytes = 256 * kHistCopies * 4;
+constexpr int kHistBytes = 257 * kHistCopies * 4;
 
 struct WindowWeights {
     float w1[kMaxWindow];
@@ -271,8 +271,9 @@ __global__ __launch_bounds__(kWG) void block_topk_kernel(int64_t d, int dbs, int
     load_block(r, xb, n, vec, wave, lane);
     uint32_t T;
     int take_eq;
-    select_threshold(r, kb, hist, sh, T, take_eq);
-    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
+    PhaseTimer pt;
+    select_threshold(r, kb, hist, sh, T, take_eq, pt, 0);
+    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 0);
     for (int j = tid; j < kb; j += kWG) {
         const int idx = sel_idx[j];
         I_row[col0 + j] = (int16_t)idx;
@@ -361,8 +362,8 @@ struct RawChunk;
 template <int C>
 struct RawChunk<RegsBF16<C>> {
     uint4 q;
-    __device__ __forceinline__ void load(const uint16_t *base, int off, int n) {
-        if (off + kChunk <= n) {
+    __device__ __forceinline__ void load(const uint16_t *base, int off, int n, bool full) {
+        if (full || off + kChunk <= n) {
             q = *reinterpret_cast<const uint4 *>(base + off);
         } else {
             uint32_t r[4] = {0, 0, 0, 0};
@@ -384,8 +385,15 @@ struct RawChunk<RegsBF16<C>> {
 template <int C>
 struct RawChunk<RegsF32<C>> {
     float v_[8];
-    __device__ __forceinline__ void load(const float *base, int off, int n) {
-        load8(base, off, n, true, v_);
+    __device__ __forceinline__ void load(const float *base, int off, int n, bool full) {
+        if (full) {
+            const float4 a = *reinterpret_cast<const float4 *>(base + off);
+            const float4 b = *reinterpret_cast<const float4 *>(base + off + 4);
+            v_[0] = a.x; v_[1] = a.y; v_[2] = a.z; v_[3] = a.w;
+            v_[4] = b.x; v_[5] = b.y; v_[6] = b.z; v_[7] = b.w;
+        } else {
+            load8(base, off, n, true, v_);
+        }
     }
     __device__ __forceinline__ void to_float(float (&v)[8]) const {
 #pragma unroll
@@ -393,12 +401,15 @@ struct RawChunk<RegsF32<C>> {
     }
 };
 
-template <class R>
-__global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
+constexpr int kPrefetchRows = 16;  // window rows held in registers when a block row fits one pass
+
+// FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
+template <class R, bool FULL>
+__device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDesc &D,
+                                            const int64_t b, unsigned char *lds) {
     typedef typename R::elem_t elem_t;
     typedef typename R::slot_t slot_t;
     constexpr int C = R::kC;
-    extern __shared__ __align__(16) unsigned char lds[];
     uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
     uint32_t *counter = sh + 8;
     uint16_t *sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
@@ -410,18 +421,11 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
     uint16_t *coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    // which tensor, which block
-    int ti = 0;
-    for (int i = 1; i < P.n_tensors; ++i)
-        if ((int)blockIdx.x >= P.t[i].first_block) ti = i;
-    const TensorDesc &D = P.t[ti];
-    const int64_t b = (int)blockIdx.x - D.first_block;
     const int64_t d = D.d;
     const int dbs = (int)(d < P.d_block_size ? d : P.d_block_size);
     const int64_t n_full = d / dbs;
     const int64_t e0 = b * dbs;
-    const int n = (int)((d - e0) < dbs ? (d - e0) : dbs);
+    const int n = FULL ? C * 2048 : (int)((d - e0) < dbs ? (d - e0) : dbs);
     const int kb = b < n_full ? D.k_many : D.k_few;
     const int64_t col0 = b * D.k_many;
     const elem_t *g = reinterpret_cast<const elem_t *>(D.g) + e0;
@@ -429,53 +433,83 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
     uint8_t *err = D.err + (e0 >> 1);
     const int q_shift = P.q_shift;
     const int ql = 1 << (q_shift - 3);  // lanes per quantisation block
+    PhaseTimer pt;
+    pt.begin();
 
-    // ---- parameters: issued first, consumed last
+    // ---- parameters and the older window rows are requested first and consumed last, so
+    //      their memory latency hides behind the selection and quantisation work
     RawChunk<R> praw[C];
 #pragma unroll
-    for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n);
-
-    // ---- a = g + Qinv(e), rounded to the element type (MA:190)
-    R r;
+    for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
+    const int rows = P.W.rows;
+    const bool fast_window = kb <= kWG && rows <= kPrefetchRows && P.L.sub_len >= n;
+    uint32_t ent[kPrefetchRows];  // (value << 16) | index of this thread's entry in each row
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-        const int off = chunk_off<C>(wave, c, lane);
-        float v[8];
-        load8(g, off, n, true, v);
-        uint32_t cw = 0;
-        float mn = 0.0f, mx = 0.0f;
-        if (off < n) {
-            if (off + kChunk <= n) {
-                cw = *reinterpret_cast<const uint32_t *>(err + (off >> 1));
-            } else {
-                const int nbytes = (n - off + 1) >> 1;
-                for (int j = 0; j < nbytes; ++j) cw |= (uint32_t)err[(off >> 1) + j] << (8 * j);
-            }
-            const int64_t qb = (e0 + off) >> q_shift;
-            mn = bf2f(D.mn[qb]);
-            mx = bf2f(D.mx[qb]);
-        }
-        const float u = (mx - mn) / 15.0f;
-#pragma unroll
-        for (int e = 0; e < kChunk; ++e) {
-            const uint32_t code = (cw >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
-            float deq = (float)code * u;
-            deq = deq + mn;
-            v[e] = v[e] + deq;
-        }
-        if (off + kChunk > n) {
-#pragma unroll
-            for (int e = 0; e < kChunk; ++e)
-                if (off + e >= n) v[e] = 0.0f;
-        }
-        r.set_chunk(c, v);
+    for (int row = 0; row < kPrefetchRows; ++row) {
+        ent[row] = 0;
+        if (fast_window && row < rows && row != D.row && tid < kb)
+            ent[row] = (uint32_t)(uint16_t)D.I[(int64_t)row * D.k + col0 + tid] |
+                       ((uint32_t)D.V[(int64_t)row * D.k + col0 + tid] << 16);
     }
+
+    // ---- a = g + Qinv(e), rounded to the element type (MA:190).  All loads first.
+    R r;
+    {
+        RawChunk<R> graw[C];
+        uint32_t cw[C], smn[C], smx[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            graw[c].load(g, off, n, FULL);
+            cw[c] = 0;
+            smn[c] = smx[c] = 0;
+            if (FULL || off < n) {
+                if (FULL || off + kChunk <= n) {
+                    cw[c] = *reinterpret_cast<const uint32_t *>(err + (off >> 1));
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        cw[c] |= (uint32_t)err[(off >> 1) + j] << (8 * j);
+                }
+                const int64_t qb = (e0 + off) >> q_shift;
+                smn[c] = D.mn[qb];
+                smx[c] = D.mx[qb];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float v[8];
+            graw[c].to_float(v);
+            const float mn = bf2f(smn[c]), mx = bf2f(smx[c]);
+            const float u = (mx - mn) / 15.0f;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                float deq = (float)code * u;
+                deq = deq + mn;
+                v[e] = v[e] + deq;
+            }
+            if (!FULL && off + kChunk > n) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (off + e >= n) v[e] = 0.0f;
+            }
+            r.set_chunk(c, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    launder(r);
+    pt.mark(0);
 
     // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214)
     uint32_t T;
     int take_eq;
-    select_threshold(r, kb, hist, sh, T, take_eq);
-    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
+    select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
+    launder(r);
+    pt.mark(7);
+    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
+    launder(r);
     {
         int16_t *Irow = D.I + (int64_t)D.row * D.k + col0;
         uint16_t *Vrow = D.V + (int64_t)D.row * D.k + col0;
@@ -484,6 +518,7 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
             Vrow[j] = sel_val[j];
         }
     }
+    pt.mark(10);
 
     // ---- residual statistics (MA:217-228) and 4-bit codes (MA:231)
 #pragma unroll
@@ -494,18 +529,14 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
             x[e] = r.val(c, e);
-            if (off + e < n) {
-                mn = x[e] < mn ? x[e] : mn;
-                mx = x[e] > mx ? x[e] : mx;
+            if (FULL || off + e < n) {
+                mn = __builtin_fminf(mn, x[e]);
+                mx = __builtin_fmaxf(mx, x[e]);
             }
         }
-        for (int s = 1; s < ql; s <<= 1) {
-            const float a = __shfl_xor(mn, s, kWave), c2 = __shfl_xor(mx, s, kWave);
-            mn = a < mn ? a : mn;
-            mx = c2 > mx ? c2 : mx;
-        }
+        group_minmax(mn, mx, ql);
         const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
-        if (off < n) {
+        if (FULL || off < n) {
             if ((lane & (ql - 1)) == 0) {
                 const int64_t qb = (e0 + off) >> q_shift;
                 D.mn[qb] = (uint16_t)mnb;
@@ -514,45 +545,132 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
             const float mnf = bf2f(mnb), mxf = bf2f(mxb);
             const float u = (mxf - mnf) / 15.0f;
             const bool ok = u != 0.0f && isfinite(u);
+            const Divisor dv = make_divisor(u);
             uint32_t cw = 0;
+            if (dv.safe) {
+                // codes gathered as small exact floats: two 16-bit halves, nibble order
+                // (e0 e1)(e2 e3) | (e4 e5)(e6 e7) with the even element in the high nibble
+                float cf[8];
+                const float lim = 32.0f * u;
 #pragma unroll
-            for (int e = 0; e < kChunk; ++e) {
-                const uint32_t code = (off + e < n) ? quant_code(x[e], mnf, u, ok) : 0u;
-                cw |= code << (8 * (e >> 1) + ((e & 1) ? 0 : 4));
+                for (int e = 0; e < kChunk; ++e) {
+                    float y = x[e] - mnf;
+                    if (!R::kBF16) y = __builtin_amdgcn_fmed3f(y, -lim, lim);
+                    float v = div_shared(y, dv);
+                    v = floorf(v + 0.5f);
+                    if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+                    cf[e] = (FULL || off + e < n) ? v : 0.0f;
+                }
+                float lo = cf[2];
+                lo = __builtin_fmaf(lo, 16.0f, cf[3]);
+                lo = __builtin_fmaf(lo, 16.0f, cf[0]);
+                lo = __builtin_fmaf(lo, 16.0f, cf[1]);
+                float hi = cf[6];
+                hi = __builtin_fmaf(hi, 16.0f, cf[7]);
+                hi = __builtin_fmaf(hi, 16.0f, cf[4]);
+                hi = __builtin_fmaf(hi, 16.0f, cf[5]);
+                cw = (uint32_t)lo | ((uint32_t)hi << 16);
+            } else {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    const uint32_t code =
+                        (FULL || off + e < n) ? quant_code(x[e], mnf, u, ok) : 0u;
+                    cw |= code << (8 * (e >> 1) + ((e & 1) ? 0 : 4));
+                }
             }
-            if (off + kChunk <= n) {
+            if (FULL || off + kChunk <= n) {
                 *reinterpret_cast<uint32_t *>(err + (off >> 1)) = cw;
             } else {
                 const int nbytes = (n - off + 1) >> 1;
                 for (int j = 0; j < nbytes; ++j) err[(off >> 1) + j] = (uint8_t)(cw >> (8 * j));
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
+    pt.mark(11);
 
     // ---- Adam direction from the window (MA:277-291); the slot cells end up holding the
     //      update's bits, 0 where no window row names the coordinate
     __syncthreads();  // the histogram's LDS is reused below
-    for (int i = tid; i < P.L.slot_cells; i += kWG) slot[i] = 0;
-    WindowView wv;
-    wv.I = D.I + col0;
-    wv.V = D.V + col0;
-    wv.k = D.k;
-    wv.rows = P.W.rows;
-    wv.cur_row = D.row;
-    wv.cur_idx = sel_idx;
-    wv.cur_val = sel_val;
-    wv.w1 = P.W.w1;
-    wv.w2 = P.W.w2;
-    for (int lo = 0; lo < n; lo += P.L.sub_len) {
-        const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
-        window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
-        const int cnt = (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
-        for (int s = tid; s < cnt; s += kWG) {
-            const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
-            slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+    for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
+        reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+    if (fast_window) {
+        // One entry per thread and row.  Entry (row, tid) owns row*kb + tid of z1 / z2 / coord;
+        // the first entry (in row order) to name a coordinate becomes its owner and later
+        // rows add into the owner's sums.  Rows are separated by barriers and a row never
+        // names a coordinate twice, so the sums are formed in row order.
+        __syncthreads();
+        pt.mark(12);
+#pragma unroll
+        for (int row = 0; row < kPrefetchRows; ++row) {
+            if (row < rows) {
+                uint32_t en = ent[row];
+                if (row == D.row && tid < kb)
+                    en = (uint32_t)sel_idx[tid] | ((uint32_t)sel_val[tid] << 16);
+                const int idx = (int)(en & 0xffffu);
+                const uint32_t vb = en >> 16;
+                // +-0 values add nothing and are skipped (the rows of a fresh window are all
+                // (index 0, value 0)); idx < n also keeps a corrupt index inside the block
+                const bool active = tid < kb && idx < n && (vb & 0x7fffu) != 0;
+                const int own = row * kb + tid;
+                if (tid < kb) {
+                    const float v = bf2f(vb);
+                    const float a1 = P.W.w1[row] * v;
+                    const float vv = v * v;
+                    const float a2 = P.W.w2[row] * vv;
+                    uint32_t owner_idx = 0xffffu;
+                    if (active) {
+                        const uint32_t s = slot[idx];
+                        if (s == 0) {
+                            slot[idx] = (slot_t)(own + 1);
+                            z1[own] = 0.0f + a1;
+                            z2[own] = 0.0f + a2;
+                            owner_idx = (uint32_t)idx;
+                        } else {
+                            z1[s - 1] = z1[s - 1] + a1;
+                            z2[s - 1] = z2[s - 1] + a2;
+                        }
+                    }
+                    coord[own] = (uint16_t)owner_idx;
+                }
+                __syncthreads();
+            }
+        }
+        pt.mark(13);
+        const int entries = rows * kb;
+        for (int s = tid; s < entries; s += kWG) {
+            const uint32_t ci = coord[s];
+            if (ci != 0xffffu) {
+                const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
+                slot[ci] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+            }
         }
         __syncthreads();
+        pt.mark(14);
+    } else {
+        WindowView wv;
+        wv.I = D.I + col0;
+        wv.V = D.V + col0;
+        wv.k = D.k;
+        wv.rows = rows;
+        wv.cur_row = D.row;
+        wv.cur_idx = sel_idx;
+        wv.cur_val = sel_val;
+        wv.w1 = P.W.w1;
+        wv.w2 = P.W.w2;
+        for (int lo = 0; lo < n; lo += P.L.sub_len) {
+            const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+            window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
+            const int cnt =
+                (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
+            for (int s = tid; s < cnt; s += kWG) {
+                const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
+                slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+            }
+            __syncthreads();
+        }
     }
+    pt.mark(15);
 
     // ---- p = p * (1 - lr*wd) (MA:234-235); p += -lr * u (MA:304)
     const float neg_lr = D.neg_lr, decay = D.decay;
@@ -560,7 +678,7 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         const int off = chunk_off<C>(wave, c, lane);
-        if (off < n) {
+        if (FULL || off < n) {
             float pv[8], uv[8];
             praw[c].to_float(pv);
             if (R::kBF16) {
@@ -579,19 +697,40 @@ __global__ __launch_bounds__(kWG) void fused_step_kernel(FusedParams P) {
                 uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
                 uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
             }
+            if (apply_decay) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    pv[e] = pv[e] * decay;
+                    if (R::kBF16) pv[e] = bf2f(f2bf(pv[e]));
+                }
+            }
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                float x = pv[e];
-                if (apply_decay) {
-                    x = x * decay;
-                    if (R::kBF16) x = bf2f(f2bf(x));
-                }
                 const float prod = neg_lr * uv[e];
-                pv[e] = x + prod;
+                pv[e] = pv[e] + prod;
             }
-            store8(p, off, n, true, pv);
+            store8(p, off, FULL ? 0x7fffffff : n, true, pv);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
+    pt.mark(16);
+}
+
+template <class R, int MIN_WAVES>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    // which tensor, which block
+    int ti = 0;
+    for (int i = 1; i < P.n_tensors; ++i)
+        if ((int)blockIdx.x >= P.t[i].first_block) ti = i;
+    const TensorDesc &D = P.t[ti];
+    const int64_t b = (int)blockIdx.x - D.first_block;
+    const int64_t dbs = D.d < P.d_block_size ? D.d : P.d_block_size;
+    const int64_t left = D.d - b * dbs;
+    if (dbs == R::kC * 2048 && left >= dbs)
+        fused_block<R, true>(P, D, b, lds);
+    else
+        fused_block<R, false>(P, D, b, lds);
 }
 
 // =============================================================================================
@@ -687,9 +826,9 @@ template <template <int> class RT>
 static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
 #define MA_FUSED_CASE(CC)                                                     \
     case CC: {                                                                \
-        int rc = allow_big_lds(fused_step_kernel<RT<CC>>, lds_bytes);         \
+        int rc = allow_big_lds(fused_step_kernel<RT<CC>, 2>, lds_bytes);      \
         if (rc) return rc;                                                    \
-        fused_step_kernel<RT<CC>><<<grid, kWG, lds_bytes, s>>>(P);            \
+        fused_step_kernel<RT<CC>, 2><<<grid, kWG, lds_bytes, s>>>(P);         \
         return launch_status();                                               \
     }
     switch (C) {
@@ -922,6 +1061,12 @@ int ma_compute_microadam_update(int blocks, int threads, int carveout, int64_t t
     }
     return launch_status();
 }
+
+#ifdef MA_PHASE_TIMING
+int ma_debug_set_phase_buffer(void *buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_phase_buf), &buf, sizeof(buf));
+}
+#endif
 
 int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
     return fused_check(tensor, hyper);
