@@ -331,6 +331,191 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
     take_eq = need;
 }
 
+// ---- top-k through chunk maxima (bf16, k much smaller than the block) ---------------------------
+//
+// Every lane keeps only the largest key of each of its 8-element chunks.  If L is the kb-th
+// largest chunk maximum, at least kb chunks hold an element >= L, so the kb-th largest element
+// T satisfies T >= L: every member of the top-k has key >= L.  For k = 1 % of the block about
+// 1.04 k elements pass that test, and the exact top-k (magnitude first, lowest index on ties)
+// is then taken among those few candidates by rank.  The block itself waits in LDS meanwhile.
+
+// largest 15-bit magnitude key among the 8 bf16 values of a chunk
+__device__ __forceinline__ uint32_t chunk_max_key(const uint32_t (&w)[4]) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    us2 k0 = __builtin_bit_cast(us2, w[0] & 0x7fff7fffu);
+    us2 k1 = __builtin_bit_cast(us2, w[1] & 0x7fff7fffu);
+    us2 k2 = __builtin_bit_cast(us2, w[2] & 0x7fff7fffu);
+    us2 k3 = __builtin_bit_cast(us2, w[3] & 0x7fff7fffu);
+    k0 = __builtin_elementwise_max(k0, k1);
+    k2 = __builtin_elementwise_max(k2, k3);
+    k0 = __builtin_elementwise_max(k0, k2);
+    const uint32_t m = __builtin_bit_cast(uint32_t, k0);
+    const uint32_t lo = m & 0xffffu, hi = m >> 16;
+    return lo > hi ? lo : hi;
+}
+
+constexpr int kSmallCopies = 8;
+constexpr int kSmallHistWords = 257 * kSmallCopies;
+
+// kb-th largest of the N * 256 keys (15 bits each) held N per thread; 1 <= kb <= N * 256.
+// hist: kSmallHistWords words, sh: 8 words.  Ends with a barrier.
+template <int N>
+__device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], int kb,
+                                                     uint32_t *hist, uint32_t *sh) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t prefix = 0, pmask = 0;
+    int need = kb;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int shift = pass == 0 ? 7 : 0;
+        const int nb = pass == 0 ? 256 : 128;
+        const uint32_t dm = nb - 1;
+        for (int i = tid; i < nb * kSmallCopies / 4; i += kWG)
+            reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const uint32_t bin = (v[i] & pmask) == prefix ? ((v[i] >> shift) & dm) : 256u;
+            atomicAdd(&hist[bin * kSmallCopies + (lane & (kSmallCopies - 1))], 1u);
+        }
+        __syncthreads();
+        const int bin = nb - 1 - tid;
+        uint32_t cnt = 0;
+        if (bin >= 0) {
+            const uint4 a = reinterpret_cast<const uint4 *>(hist)[bin * 2];
+            const uint4 b = reinterpret_cast<const uint4 *>(hist)[bin * 2 + 1];
+            cnt = a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
+        }
+        const uint32_t incl = wg_incl_scan(cnt, sh, lane, wave);
+        const uint32_t excl = incl - cnt;
+        if (bin >= 0 && excl < (uint32_t)need && (uint32_t)need <= incl) {
+            sh[4] = (uint32_t)bin;
+            sh[5] = (uint32_t)need - excl;
+        }
+        __syncthreads();
+        prefix |= sh[4] << shift;
+        pmask |= dm << shift;
+        need = (int)sh[5];
+    }
+    __syncthreads();
+    return prefix;
+}
+
+constexpr int kCandPerWave = 128;  // candidate slots per wave; more than that falls back
+
+// The fast top-k of a full bf16 block.  `park` (2048*C uint16 cells) receives the block;
+// on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
+// magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false
+// (a wave found more candidates than it has room for: heavy ties) r is reloaded unchanged.
+//   hist: kSmallHistWords + 4*kCandPerWave words; sh: 16 words.  1 <= kb <= 256.
+template <class R>
+__device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uint32_t *hist,
+                                               uint32_t *sh, uint16_t *sel_idx,
+                                               uint16_t *sel_val) {
+    constexpr int C = R::kC;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t *cand = hist + kSmallHistWords;
+    uint32_t cmax[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int off = chunk_off<C>(wave, c, lane);
+        *reinterpret_cast<uint4 *>(park + off) =
+            make_uint4(r.w[c][0], r.w[c][1], r.w[c][2], r.w[c][3]);
+        cmax[c] = chunk_max_key(r.w[c]);
+    }
+    const uint32_t L = select_kth_key15<C>(cmax, kb, hist, sh);
+
+    // candidates: every element with key >= L, wave by wave into the wave's own list
+    uint32_t todo = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) todo |= (cmax[c] >= L ? 1u : 0u) << c;
+    uint32_t *mine = cand + wave * kCandPerWave;
+    uint32_t filled = 0;  // wave-uniform
+    while (__ballot(todo != 0) != 0) {
+        const bool has = todo != 0;
+        const int c = has ? __ffs(todo) - 1 : 0;
+        todo &= todo - 1;
+        const int off = ((wave * C + c) * kWave + lane) * kChunk;
+        const uint4 q = *reinterpret_cast<const uint4 *>(park + off);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        uint32_t m8 = 0;
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            const uint32_t key = (e & 1) ? ((w[e >> 1] >> 16) & 0x7fffu) : (w[e >> 1] & 0x7fffu);
+            m8 |= (key >= L ? 1u : 0u) << e;
+        }
+        if (!has) m8 = 0;
+        const uint32_t cnt = __popc(m8);
+        const uint32_t incl = wave_incl_scan(cnt, lane);
+        uint32_t pos = filled + incl - cnt;
+        filled += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        while (m8) {
+            const int e = __ffs(m8) - 1;
+            m8 &= m8 - 1;
+            const uint32_t pair = (e >> 1) == 0 ? w[0] : (e >> 1) == 1 ? w[1] : (e >> 1) == 2 ? w[2] : w[3];
+            const uint32_t key = (pair >> ((e & 1) * 16)) & 0x7fffu;
+            if (pos < (uint32_t)kCandPerWave) mine[pos] = (key << 15) | (uint32_t)(32767 - (off + e));
+            ++pos;
+        }
+    }
+    // pad the wave's list to a multiple of 4 with zeros (never greater than a candidate)
+    if (lane < 4 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
+    if (lane == 0) sh[12 + wave] = filled;
+    __syncthreads();
+    uint32_t cnts[kWaves];
+    bool ok = true;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        cnts[w] = sh[12 + w];
+        ok = ok && cnts[w] <= (uint32_t)kCandPerWave;
+    }
+    if (ok) {
+        // rank of each candidate among all candidates: composites are distinct, larger wins
+        const int total = (int)(cnts[0] + cnts[1] + cnts[2] + cnts[3]);
+        for (int base = 0; base < total; base += kWG) {
+            int i = base + tid;
+            uint32_t my = 0;
+            bool have = false;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                if (!have && i >= 0 && i < (int)cnts[w]) {
+                    my = cand[w * kCandPerWave + i];
+                    have = true;
+                }
+                i -= (int)cnts[w];
+            }
+            uint32_t rank = 0;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const uint4 *seg = reinterpret_cast<const uint4 *>(cand + w * kCandPerWave);
+                const int quads = ((int)cnts[w] + 3) >> 2;
+                for (int j = 0; j < quads; ++j) {
+                    const uint4 o = seg[j];
+                    rank += (o.x > my ? 1u : 0u) + (o.y > my ? 1u : 0u) + (o.z > my ? 1u : 0u) +
+                            (o.w > my ? 1u : 0u);
+                }
+            }
+            if (have && rank < (uint32_t)kb) {
+                const uint32_t idx = 32767u - (my & 0x7fffu);
+                sel_idx[rank] = (uint16_t)idx;
+                sel_val[rank] = park[idx];
+                park[idx] = 0;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int off = chunk_off<C>(wave, c, lane);
+        const uint4 q = *reinterpret_cast<const uint4 *>(park + off);
+        r.w[c][0] = q.x;
+        r.w[c][1] = q.y;
+        r.w[c][2] = q.z;
+        r.w[c][3] = q.w;
+    }
+    return ok;
+}
+
 // ---- ordered compaction ------------------------------------------------------------------------
 //
 // Selects every entry with key > T plus the first `take_eq` entries (in index order) with

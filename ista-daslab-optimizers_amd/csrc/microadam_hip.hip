@@ -503,13 +503,24 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
     pt.mark(0);
 
     // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214)
-    uint32_t T;
-    int take_eq;
-    select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
-    launder(r);
-    pt.mark(7);
-    compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
-    launder(r);
+    bool topk_done = false;
+    if constexpr (FULL && R::kBF16) {
+        if (kb <= kWG) {
+            topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
+                                       sel_idx, sel_val);
+            launder(r);
+            pt.mark(7);
+        }
+    }
+    if (!topk_done) {
+        uint32_t T;
+        int take_eq;
+        select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
+        launder(r);
+        pt.mark(7);
+        compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
+        launder(r);
+    }
     {
         int16_t *Irow = D.I + (int64_t)D.row * D.k + col0;
         uint16_t *Vrow = D.V + (int64_t)D.row * D.k + col0;

@@ -183,6 +183,20 @@ def unpack_codes(xq, d):
     return out[:d]
 
 
+def canonical_window(I, V, k_block_size_many):
+    """Window rows with the entries of every block sorted by index.
+
+    The order of the k_block entries inside a block of a row carries no meaning (the reference
+    takes them from torch.topk(sorted=False), micro_adam.py:193-200, and the Adam statistics do
+    not depend on it), so two states are the same window iff they agree after this sort."""
+    I = np.asarray(I)
+    V = np.asarray(V).reshape(I.shape)
+    blk = (np.arange(I.shape[1]) // k_block_size_many).astype(np.int64)
+    key = blk[None, :] * 65536 + I.astype(np.int64)
+    order = np.argsort(key, axis=1, kind="stable")
+    return np.take_along_axis(I, order, axis=1), np.take_along_axis(V, order, axis=1)
+
+
 # ---- optimizer-shaped driver -----------------------------------------------------
 
 class OracleMicroAdam:

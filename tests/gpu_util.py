@@ -28,9 +28,16 @@ def state_snapshot(st):
 
 
 def assert_state_equal(gst, ost, ctx=""):
-    """Bit-exact comparison of a GPU optimizer state with the oracle's."""
+    """Bit-exact comparison of a GPU optimizer state with the oracle's.  The window is compared
+    as index sets with their values: entries of a block row are sorted by index first, since
+    their order inside the block is unspecified (torch.topk(sorted=False) in the reference)."""
+    import microadam_oracle as oracle
     snap = state_snapshot(gst)
     assert gst["index"] == ost["index"], ctx
+    km = ost["k_block_size_many"]
+    snap["I"], snap["V"] = oracle.canonical_window(snap["I"], snap["V"], km)
+    ost = dict(ost)
+    ost["I"], ost["V"] = oracle.canonical_window(ost["I"], ost["V"], km)
     for key in ("I", "V", "error", "min_vals", "max_vals"):
         a, b = snap[key], np.asarray(ost[key]).reshape(snap[key].shape)
         if not np.array_equal(a, b):
