@@ -38,7 +38,8 @@ struct PhaseTimer {
 #else
 struct PhaseTimer {
     __device__ __forceinline__ void begin() {}
-    __device__ __forceinline__ void mark(int) {}
+    // leaves a comment in the assembly listing so that instruction counts can be read per phase
+    __device__ __forceinline__ void mark(int i) { asm volatile("; phase mark %0" ::"n"(i)); }
 };
 #endif
 
@@ -83,33 +84,49 @@ __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane) {
     return v;
 }
 
+// min / max of two numbers that are not NaN, one instruction each.  (fminf / fmaxf, and the
+// median-of-three builtin with an infinity, are lowered with a re-quieting of both operands.)
+__device__ __forceinline__ float fmin_raw(float a, float b) {
+    float d;
+    asm("v_min_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+__device__ __forceinline__ float fmax_raw(float a, float b) {
+    float d;
+    asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_perm(float v) {
     return __int_as_float(
         __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
-// min / max over aligned groups of `ql` lanes (a power of two), result in every lane
-__device__ __forceinline__ void group_minmax(float &mn, float &mx, int ql) {
+// min / max over aligned groups of `ql` lanes (a power of two), result in every lane.
+// QL > 0 fixes the group size at compile time; QL == 0 takes it from `ql`.
+template <int QL>
+__device__ __forceinline__ void group_minmax(float &mn, float &mx, int ql_runtime) {
+    const int ql = QL > 0 ? QL : ql_runtime;
     if (ql >= 2) {
-        mn = __builtin_fminf(mn, dpp_perm<0xB1>(mn));  // quad_perm [1,0,3,2]
-        mx = __builtin_fmaxf(mx, dpp_perm<0xB1>(mx));
+        mn = fmin_raw(mn, dpp_perm<0xB1>(mn));  // quad_perm [1,0,3,2]
+        mx = fmax_raw(mx, dpp_perm<0xB1>(mx));
     }
     if (ql >= 4) {
-        mn = __builtin_fminf(mn, dpp_perm<0x4E>(mn));  // quad_perm [2,3,0,1]
-        mx = __builtin_fmaxf(mx, dpp_perm<0x4E>(mx));
+        mn = fmin_raw(mn, dpp_perm<0x4E>(mn));  // quad_perm [2,3,0,1]
+        mx = fmax_raw(mx, dpp_perm<0x4E>(mx));
     }
     if (ql >= 8) {
-        mn = __builtin_fminf(mn, dpp_perm<0x141>(mn));  // row_half_mirror
-        mx = __builtin_fmaxf(mx, dpp_perm<0x141>(mx));
+        mn = fmin_raw(mn, dpp_perm<0x141>(mn));  // row_half_mirror
+        mx = fmax_raw(mx, dpp_perm<0x141>(mx));
     }
     if (ql >= 16) {
-        mn = __builtin_fminf(mn, dpp_perm<0x140>(mn));  // row_mirror
-        mx = __builtin_fmaxf(mx, dpp_perm<0x140>(mx));
+        mn = fmin_raw(mn, dpp_perm<0x140>(mn));  // row_mirror
+        mx = fmax_raw(mx, dpp_perm<0x140>(mx));
     }
     for (int s = 16; s < ql; s <<= 1) {
-        mn = __builtin_fminf(mn, __shfl_xor(mn, s, kWave));
-        mx = __builtin_fmaxf(mx, __shfl_xor(mx, s, kWave));
+        mn = fmin_raw(mn, __shfl_xor(mn, s, kWave));
+        mx = fmax_raw(mx, __shfl_xor(mx, s, kWave));
     }
 }
 
@@ -672,12 +689,12 @@ __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, 
 // y / u, correctly rounded, with the refinement of 1/u paid once.  This is the fp32 division
 // expansion of the compiler (reciprocal, one Newton step, quotient, two fused residual
 // corrections) without its operand scaling and special-case fix-up, so it equals IEEE division
-// bit for bit whenever those would be no-ops: u normal and away from the ends of the exponent
-// range (`safe`), and the quotient neither overflowing nor denormal.  Callers keep |y| within a
-// few multiples of 16 u, and a quotient below 2^-30 is only ever compared with 1/2.
+// bit for bit whenever those would be no-ops: u normal with a biased exponent in [32, 222]
+// (callers scale u and y by an exact power of two to get there), and the quotient neither
+// overflowing nor denormal.  Callers keep |y| within a few multiples of 16 u, and a quotient
+// below 2^-30 is only ever compared with 1/2.
 struct Divisor {
     float u, r;
-    bool safe;
 };
 
 __device__ __forceinline__ Divisor make_divisor(float u) {
@@ -686,8 +703,6 @@ __device__ __forceinline__ Divisor make_divisor(float u) {
     const float r0 = __builtin_amdgcn_rcpf(u);
     const float e = __builtin_fmaf(-u, r0, 1.0f);
     d.r = __builtin_fmaf(e, r0, r0);
-    const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
-    d.safe = ex >= 32u && ex <= 222u;
     return d;
 }
 
@@ -697,6 +712,14 @@ __device__ __forceinline__ float div_shared(float y, const Divisor &d) {
     const float q1 = __builtin_fmaf(e1, d.r, q0);
     const float e2 = __builtin_fmaf(-d.u, q1, y);
     return __builtin_fmaf(e2, d.r, q1);
+}
+
+// x / 15 for the quantisation step u = (max - min) / 15: the shared-divisor sequence when the
+// range is comfortably normal, the compiler's full division otherwise.
+__device__ __forceinline__ float div15(float x, const Divisor &d15) {
+    const uint32_t ex = (__float_as_uint(x) >> 23) & 0xffu;
+    if (ex - 32u <= 190u) return div_shared(x, d15);
+    return x / 15.0f;
 }
 
 __device__ __forceinline__ float adam_direction(float z1, float z2, float s1, float s2,

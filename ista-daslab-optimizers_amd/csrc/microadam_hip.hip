@@ -404,7 +404,7 @@ struct RawChunk<RegsF32<C>> {
 constexpr int kPrefetchRows = 16;  // window rows held in registers when a block row fits one pass
 
 // FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
-template <class R, bool FULL>
+template <class R, bool FULL, int QL>
 __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDesc &D,
                                             const int64_t b, unsigned char *lds) {
     typedef typename R::elem_t elem_t;
@@ -431,8 +431,9 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
     const elem_t *g = reinterpret_cast<const elem_t *>(D.g) + e0;
     elem_t *p = reinterpret_cast<elem_t *>(D.p) + e0;
     uint8_t *err = D.err + (e0 >> 1);
-    const int q_shift = P.q_shift;
+    const int q_shift = QL > 0 ? (QL == 4 ? 5 : 6) : P.q_shift;
     const int ql = 1 << (q_shift - 3);  // lanes per quantisation block
+    const Divisor d15 = make_divisor(15.0f);
     PhaseTimer pt;
     pt.begin();
 
@@ -482,7 +483,7 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
             float v[8];
             graw[c].to_float(v);
             const float mn = bf2f(smn[c]), mx = bf2f(smx[c]);
-            const float u = (mx - mn) / 15.0f;
+            const float u = div15(mx - mn, d15);
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
                 const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
@@ -541,54 +542,63 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
         for (int e = 0; e < kChunk; ++e) {
             x[e] = r.val(c, e);
             if (FULL || off + e < n) {
-                mn = __builtin_fminf(mn, x[e]);
-                mx = __builtin_fmaxf(mx, x[e]);
+                mn = fmin_raw(mn, x[e]);
+                mx = fmax_raw(mx, x[e]);
             }
         }
-        group_minmax(mn, mx, ql);
+        group_minmax<QL>(mn, mx, ql);
         const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
         if (FULL || off < n) {
             if ((lane & (ql - 1)) == 0) {
-                const int64_t qb = (e0 + off) >> q_shift;
+                const uint32_t qb = (uint32_t)(e0 >> q_shift) + ((uint32_t)off >> q_shift);
                 D.mn[qb] = (uint16_t)mnb;
                 D.mx[qb] = (uint16_t)mxb;
             }
             const float mnf = bf2f(mnb), mxf = bf2f(mxb);
-            const float u = (mxf - mnf) / 15.0f;
-            const bool ok = u != 0.0f && isfinite(u);
-            const Divisor dv = make_divisor(u);
-            uint32_t cw = 0;
-            if (dv.safe) {
-                // codes gathered as small exact floats: two 16-bit halves, nibble order
-                // (e0 e1)(e2 e3) | (e4 e5)(e6 e7) with the even element in the high nibble
-                float cf[8];
-                const float lim = 32.0f * u;
+            const float u = div15(mxf - mnf, d15);
+            const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
+            const float lim = 32.0f * u;
+            float y[8];
 #pragma unroll
-                for (int e = 0; e < kChunk; ++e) {
-                    float y = x[e] - mnf;
-                    if (!R::kBF16) y = __builtin_amdgcn_fmed3f(y, -lim, lim);
-                    float v = div_shared(y, dv);
-                    v = floorf(v + 0.5f);
-                    if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
-                    cf[e] = (FULL || off + e < n) ? v : 0.0f;
-                }
-                float lo = cf[2];
-                lo = __builtin_fmaf(lo, 16.0f, cf[3]);
-                lo = __builtin_fmaf(lo, 16.0f, cf[0]);
-                lo = __builtin_fmaf(lo, 16.0f, cf[1]);
-                float hi = cf[6];
-                hi = __builtin_fmaf(hi, 16.0f, cf[7]);
-                hi = __builtin_fmaf(hi, 16.0f, cf[4]);
-                hi = __builtin_fmaf(hi, 16.0f, cf[5]);
-                cw = (uint32_t)lo | ((uint32_t)hi << 16);
-            } else {
-#pragma unroll
-                for (int e = 0; e < kChunk; ++e) {
-                    const uint32_t code =
-                        (FULL || off + e < n) ? quant_code(x[e], mnf, u, ok) : 0u;
-                    cw |= code << (8 * (e >> 1) + ((e & 1) ? 0 : 4));
-                }
+            for (int e = 0; e < kChunk; ++e) {
+                y[e] = x[e] - mnf;
+                // fp32 data may leave the bf16-rounded range; anything beyond +-32 u clamps
+                // to an end code either way
+                if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
             }
+            bool ok = true;
+            float us = u;
+            if (ex - 32u > 190u) {
+                // zero / non-finite range: code 0.  Otherwise bring the divisor into the
+                // exponent range where div_shared is exact by an exact power-of-two scaling
+                // of divisor and numerators; the quotient does not change.
+                ok = u != 0.0f && isfinite(u);
+                const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
+                us = ok ? u * sc : 1.0f;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
+            }
+            const Divisor dv = make_divisor(us);
+            // codes gathered as small exact floats: two 16-bit halves, nibble order
+            // (e0 e1)(e2 e3) | (e4 e5)(e6 e7) with the even element in the high nibble
+            float cf[8];
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                float v = div_shared(y[e], dv);
+                v = floorf(v + 0.5f);
+                if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+                cf[e] = (FULL || off + e < n) ? v : 0.0f;
+            }
+            float lo = cf[2];
+            lo = __builtin_fmaf(lo, 16.0f, cf[3]);
+            lo = __builtin_fmaf(lo, 16.0f, cf[0]);
+            lo = __builtin_fmaf(lo, 16.0f, cf[1]);
+            float hi = cf[6];
+            hi = __builtin_fmaf(hi, 16.0f, cf[7]);
+            hi = __builtin_fmaf(hi, 16.0f, cf[4]);
+            hi = __builtin_fmaf(hi, 16.0f, cf[5]);
+            uint32_t cw = (uint32_t)lo | ((uint32_t)hi << 16);
+            cw = ok ? cw : 0u;
             if (FULL || off + kChunk <= n) {
                 *reinterpret_cast<uint32_t *>(err + (off >> 1)) = cw;
             } else {
@@ -727,9 +737,22 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
     pt.mark(16);
 }
 
-template <class R, int MIN_WAVES>
+// QL: lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any q.
+template <class R, int MIN_WAVES, int QL>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
+#ifdef MA_STAGGER
+    // Workgroups that start together stay in step (same work, same duration), so the
+    // memory-bound and compute-bound phases of all workgroups on the chip coincide.  The
+    // first generation breaks the step: the workgroup in the odd wave slot of each SIMD waits
+    // about half a block time before it starts.
+    if (blockIdx.x < (unsigned)MA_STAGGER_FIRST) {
+        const unsigned hw = __builtin_amdgcn_s_getreg((3 << 11) | 4);  // HW_ID[3:0] = wave slot
+        if (hw & 1u) {
+            for (int i = 0; i < MA_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
+        }
+    }
+#endif
     // which tensor, which block
     int ti = 0;
     for (int i = 1; i < P.n_tensors; ++i)
@@ -738,10 +761,14 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     const int64_t b = (int)blockIdx.x - D.first_block;
     const int64_t dbs = D.d < P.d_block_size ? D.d : P.d_block_size;
     const int64_t left = D.d - b * dbs;
+#ifdef MA_ANALYZE_FULL_ONLY  // development aid: a listing with the full-block path alone
+    fused_block<R, true, QL>(P, D, b, lds);
+#else
     if (dbs == R::kC * 2048 && left >= dbs)
-        fused_block<R, true>(P, D, b, lds);
+        fused_block<R, true, QL>(P, D, b, lds);
     else
-        fused_block<R, false>(P, D, b, lds);
+        fused_block<R, false, QL>(P, D, b, lds);
+#endif
 }
 
 // =============================================================================================
@@ -833,22 +860,25 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
     return MA_ERR_BLOCK_SIZE;
 }
 
+template <class R, int QL>
+static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    int rc = allow_big_lds(fused_step_kernel<R, 2, QL>, lds_bytes);
+    if (rc) return rc;
+    fused_step_kernel<R, 2, QL><<<grid, kWG, lds_bytes, s>>>(P);
+    return launch_status();
+}
+
 template <template <int> class RT>
 static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
-#define MA_FUSED_CASE(CC)                                                     \
-    case CC: {                                                                \
-        int rc = allow_big_lds(fused_step_kernel<RT<CC>, 2>, lds_bytes);      \
-        if (rc) return rc;                                                    \
-        fused_step_kernel<RT<CC>, 2><<<grid, kWG, lds_bytes, s>>>(P);         \
-        return launch_status();                                               \
-    }
+    // the hardware-sized block gets kernels with the quantisation group size compiled in
+    if (C == 10 && P.q_shift == 6) return launch_fused_one<RT<10>, 8>(grid, lds_bytes, s, P);
+    if (C == 10 && P.q_shift == 5) return launch_fused_one<RT<10>, 4>(grid, lds_bytes, s, P);
     switch (C) {
-        MA_FUSED_CASE(2)
-        MA_FUSED_CASE(5)
-        MA_FUSED_CASE(10)
-        MA_FUSED_CASE(16)
+        case 2: return launch_fused_one<RT<2>, 0>(grid, lds_bytes, s, P);
+        case 5: return launch_fused_one<RT<5>, 0>(grid, lds_bytes, s, P);
+        case 10: return launch_fused_one<RT<10>, 0>(grid, lds_bytes, s, P);
+        case 16: return launch_fused_one<RT<16>, 0>(grid, lds_bytes, s, P);
     }
-#undef MA_FUSED_CASE
     return MA_ERR_BLOCK_SIZE;
 }
 
