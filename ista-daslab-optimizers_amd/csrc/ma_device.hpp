@@ -43,6 +43,15 @@ struct PhaseTimer {
 };
 #endif
 
+// The thread id as a value the optimiser cannot see through.  Stages that run inside a
+// persistent loop derive their lane offsets from this, so that the offsets are rebuilt where
+// they are used instead of being hoisted out of the loop into long-lived registers.
+__device__ __forceinline__ int opaque_tid() {
+    int t = (int)threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
+
 // ---- scalar helpers -----------------------------------------------------------------------
 
 __device__ __forceinline__ float bf2f(uint32_t h) { return __uint_as_float(h << 16); }
@@ -297,7 +306,7 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
                                                  uint32_t &T, int &take_eq, PhaseTimer &pt,
                                                  int pt0) {
     constexpr int kPasses = R::kBF16 ? 2 : 4;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t prefix = 0, pmask = 0;
     int need = kb;
 #pragma unroll
@@ -379,7 +388,7 @@ constexpr int kSmallHistWords = 257 * kSmallCopies;
 template <int N>
 __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], int kb,
                                                      uint32_t *hist, uint32_t *sh) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t prefix = 0, pmask = 0;
     int need = kb;
 #pragma unroll
@@ -430,7 +439,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
                                                uint32_t *sh, uint16_t *sel_idx,
                                                uint16_t *sel_val) {
     constexpr int C = R::kC;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t *cand = hist + kSmallHistWords;
     uint32_t cmax[C];
 #pragma unroll
@@ -542,7 +551,7 @@ template <class R>
 __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, int kb,
                                                  uint16_t *sel_idx, uint16_t *sel_val,
                                                  uint32_t *sh, PhaseTimer &pt, int pt0) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t pre[R::kC];  // low 16: entries >= T before this lane's chunk; high 16: == T
     uint32_t run = 0;
 #pragma unroll
@@ -654,7 +663,7 @@ template <typename slot_t>
 __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, int lo, int hi,
                                                   slot_t *slot, float *z1, float *z2,
                                                   uint16_t *coord, uint32_t *counter, int cap) {
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = opaque_tid(), lane = tid & 63;
     if (tid == 0) *counter = 0;
     __syncthreads();
     const int trips = (kb + kWG - 1) / kWG;

@@ -339,11 +339,11 @@ struct TensorDesc {
     int32_t row;
     int32_t k_many;
     int32_t k_few;
-    int32_t first_block;  // first workgroup of this tensor inside the launch
+    int32_t first_block;  // first work item of this tensor inside the launch
     float neg_lr;
     float decay;
     int32_t apply_decay;
-    int32_t pad;
+    int32_t blk0;         // block of the tensor that its first work item stands for
 };
 constexpr int kTensorsPerLaunch = 24;
 
@@ -354,7 +354,7 @@ struct FusedParams {
     int32_t n_tensors;
     int32_t d_block_size;
     int32_t q_shift;  // log2(quant_block_size)
-    int32_t pad;
+    int32_t total_items;  // work items of the launch (persistent kernel)
 };
 
 template <class R>
@@ -401,63 +401,109 @@ struct RawChunk<RegsF32<C>> {
     }
 };
 
-constexpr int kPrefetchRows = 16;  // window rows held in registers when a block row fits one pass
+constexpr int kPrefetchRows = 10;  // window rows held in registers when a block row fits one pass
 
-// FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
-template <class R, bool FULL, int QL>
-__device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDesc &D,
-                                            const int64_t b, unsigned char *lds) {
-    typedef typename R::elem_t elem_t;
-    typedef typename R::slot_t slot_t;
-    constexpr int C = R::kC;
-    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
-    uint32_t *counter = sh + 8;
-    uint16_t *sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
-    uint16_t *sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
-    slot_t *slot = reinterpret_cast<slot_t *>(lds + P.L.off_slot);
-    uint32_t *hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
-    float *z1 = reinterpret_cast<float *>(lds + P.L.off_union);
-    float *z2 = z1 + P.L.z_cap;
-    uint16_t *coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
+// Where one top-k block lives: everything a stage needs to address it, copied out of the
+// launch parameters.  Wave-uniform (lives in scalar registers).
+struct BlockGeo {
+    TensorDesc D;
+    int64_t e0;    // first element
+    int64_t col0;  // first window column
+    int n;         // elements in the block
+    int kb;        // entries selected from it
+};
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t d = D.d;
+__device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64_t b) {
+    BlockGeo G;
+    G.D = P.t[ti];
+    const int64_t d = G.D.d;
     const int dbs = (int)(d < P.d_block_size ? d : P.d_block_size);
     const int64_t n_full = d / dbs;
-    const int64_t e0 = b * dbs;
-    const int n = FULL ? C * 2048 : (int)((d - e0) < dbs ? (d - e0) : dbs);
-    const int kb = b < n_full ? D.k_many : D.k_few;
-    const int64_t col0 = b * D.k_many;
-    const elem_t *g = reinterpret_cast<const elem_t *>(D.g) + e0;
-    elem_t *p = reinterpret_cast<elem_t *>(D.p) + e0;
-    uint8_t *err = D.err + (e0 >> 1);
-    const int q_shift = QL > 0 ? (QL == 4 ? 5 : 6) : P.q_shift;
-    const int ql = 1 << (q_shift - 3);  // lanes per quantisation block
-    const Divisor d15 = make_divisor(15.0f);
-    PhaseTimer pt;
-    pt.begin();
+    G.e0 = b * dbs;
+    G.n = (int)((d - G.e0) < dbs ? (d - G.e0) : dbs);
+    G.kb = b < n_full ? G.D.k_many : G.D.k_few;
+    G.col0 = b * G.D.k_many;
+    return G;
+}
 
-    // ---- parameters and the older window rows are requested first and consumed last, so
-    //      their memory latency hides behind the selection and quantisation work
-    RawChunk<R> praw[C];
-#pragma unroll
-    for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
-    const int rows = P.W.rows;
-    const bool fast_window = kb <= kWG && rows <= kPrefetchRows && P.L.sub_len >= n;
-    uint32_t ent[kPrefetchRows];  // (value << 16) | index of this thread's entry in each row
-#pragma unroll
-    for (int row = 0; row < kPrefetchRows; ++row) {
-        ent[row] = 0;
-        if (fast_window && row < rows && row != D.row && tid < kb)
-            ent[row] = (uint32_t)(uint16_t)D.I[(int64_t)row * D.k + col0 + tid] |
-                       ((uint32_t)D.V[(int64_t)row * D.k + col0 + tid] << 16);
+// The step of one block, cut into stages so that a persistent workgroup can request the next
+// block's inputs while it works on the current one.  The register arrays are members; the
+// stages say which of them they fill and which they consume.
+//   FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
+//   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
+template <class R, bool FULL, int QL>
+struct FusedBlock {
+    typedef typename R::elem_t elem_t;
+    typedef typename R::slot_t slot_t;
+    static constexpr int C = R::kC;
+
+    const FusedParams &P;
+    uint32_t *sh, *counter, *hist;
+    uint16_t *sel_idx, *sel_val, *coord;
+    slot_t *slot;
+    float *z1, *z2;
+    int tid, lane, wave, q_shift, ql;
+    Divisor d15;
+    PhaseTimer pt;
+
+    RawChunk<R> praw[C];          // parameters              load_params_window -> update
+    uint32_t entI[kPrefetchRows];  // older window rows, kept as loaded so that nothing waits
+    uint32_t entV[kPrefetchRows];  // for them before use     load_params_window -> update
+    RawChunk<R> graw[C];          // gradient                load_grad_inputs   -> dequant
+    uint32_t cw[C], smn[C], smx[C];  // 4-bit codes, stats   load_grad_inputs   -> dequant
+    R r;                          // accumulator             dequant            -> quantize
+
+    __device__ __forceinline__ FusedBlock(const FusedParams &P_, unsigned char *lds) : P(P_) {
+        sh = reinterpret_cast<uint32_t *>(lds);
+        counter = sh + 8;
+        sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
+        sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
+        slot = reinterpret_cast<slot_t *>(lds + P.L.off_slot);
+        hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
+        z1 = reinterpret_cast<float *>(lds + P.L.off_union);
+        z2 = z1 + P.L.z_cap;
+        coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
+        tid = threadIdx.x;
+        lane = tid & 63;
+        wave = tid >> 6;
+        q_shift = QL > 0 ? (QL == 4 ? 5 : 6) : P.q_shift;
+        ql = 1 << (q_shift - 3);
+        d15 = make_divisor(15.0f);
+        pt.begin();
     }
 
-    // ---- a = g + Qinv(e), rounded to the element type (MA:190).  All loads first.
-    R r;
-    {
-        RawChunk<R> graw[C];
-        uint32_t cw[C], smn[C], smx[C];
+    __device__ __forceinline__ bool fast_window(const BlockGeo &G) const {
+        return G.kb <= kWG && P.W.rows <= kPrefetchRows && P.L.sub_len >= G.n;
+    }
+
+    // ---- parameters and the older window rows: requested early, consumed last
+    __device__ __forceinline__ void load_params_window(const BlockGeo &G) {
+        const int n = FULL ? C * 2048 : G.n;
+        const elem_t *p = reinterpret_cast<const elem_t *>(G.D.p) + G.e0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
+        const bool fw = fast_window(G);
+        const int rows = P.W.rows;
+#pragma unroll
+        for (int row = 0; row < kPrefetchRows; ++row) {
+            entI[row] = entV[row] = 0;
+            if (fw && row < rows && row != G.D.row && tid < G.kb) {
+                const uint16_t *Ir =
+                    reinterpret_cast<const uint16_t *>(G.D.I) + ((int64_t)row * G.D.k + G.col0);
+                const uint16_t *Vr = G.D.V + ((int64_t)row * G.D.k + G.col0);
+                entI[row] = Ir[(unsigned)tid];
+                entV[row] = Vr[(unsigned)tid];
+            }
+        }
+    }
+
+    // ---- gradient, 4-bit error feedback and its statistics
+    __device__ __forceinline__ void load_grad_inputs(const BlockGeo &G) {
+        const int n = FULL ? C * 2048 : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+        const uint8_t *err = G.D.err + (G.e0 >> 1);
+        const uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        const uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -466,17 +512,22 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
             smn[c] = smx[c] = 0;
             if (FULL || off < n) {
                 if (FULL || off + kChunk <= n) {
-                    cw[c] = *reinterpret_cast<const uint32_t *>(err + (off >> 1));
+                    cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
                 } else {
                     const int nbytes = (n - off + 1) >> 1;
                     for (int j = 0; j < nbytes; ++j)
                         cw[c] |= (uint32_t)err[(off >> 1) + j] << (8 * j);
                 }
-                const int64_t qb = (e0 + off) >> q_shift;
-                smn[c] = D.mn[qb];
-                smx[c] = D.mx[qb];
+                const unsigned qb = (unsigned)off >> q_shift;
+                smn[c] = mnp[qb];
+                smx[c] = mxp[qb];
             }
         }
+    }
+
+    // ---- a = g + Qinv(e), rounded to the element type (MA:190)
+    __device__ __forceinline__ void dequant(const BlockGeo &G) {
+        const int n = FULL ? C * 2048 : G.n;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -499,276 +550,333 @@ __device__ __forceinline__ void fused_block(const FusedParams &P, const TensorDe
             r.set_chunk(c, v);
             __builtin_amdgcn_sched_barrier(0);
         }
+        launder(r);
+        pt.mark(0);
     }
-    launder(r);
-    pt.mark(0);
 
-    // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214)
-    bool topk_done = false;
-    if constexpr (FULL && R::kBF16) {
-        if (kb <= kWG) {
-            topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
-                                       sel_idx, sel_val);
+    // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214), window row write
+    __device__ __forceinline__ void topk_and_row(const BlockGeo &G) {
+        const int kb = G.kb;
+        bool topk_done = false;
+        if constexpr (FULL && R::kBF16) {
+            if (kb <= kWG) {
+                topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
+                                           sel_idx, sel_val);
+                launder(r);
+                pt.mark(7);
+            }
+        }
+        if (!topk_done) {
+            uint32_t T;
+            int take_eq;
+            select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
             launder(r);
             pt.mark(7);
+            compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
+            launder(r);
         }
-    }
-    if (!topk_done) {
-        uint32_t T;
-        int take_eq;
-        select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
-        launder(r);
-        pt.mark(7);
-        compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
-        launder(r);
-    }
-    {
-        int16_t *Irow = D.I + (int64_t)D.row * D.k + col0;
-        uint16_t *Vrow = D.V + (int64_t)D.row * D.k + col0;
+        int16_t *Irow = G.D.I + ((int64_t)G.D.row * G.D.k + G.col0);
+        uint16_t *Vrow = G.D.V + ((int64_t)G.D.row * G.D.k + G.col0);
         for (int j = tid; j < kb; j += kWG) {
-            Irow[j] = (int16_t)sel_idx[j];
-            Vrow[j] = sel_val[j];
+            Irow[(unsigned)j] = (int16_t)sel_idx[j];
+            Vrow[(unsigned)j] = sel_val[j];
         }
+        pt.mark(10);
     }
-    pt.mark(10);
 
     // ---- residual statistics (MA:217-228) and 4-bit codes (MA:231)
+    __device__ __forceinline__ void quantize(const BlockGeo &G) {
+        const int n = FULL ? C * 2048 : G.n;
+        uint8_t *err = G.D.err + (G.e0 >> 1);
+        uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-        const int off = chunk_off<C>(wave, c, lane);
-        float x[8];
-        float mn = INFINITY, mx = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < kChunk; ++e) {
-            x[e] = r.val(c, e);
-            if (FULL || off + e < n) {
-                mn = fmin_raw(mn, x[e]);
-                mx = fmax_raw(mx, x[e]);
-            }
-        }
-        group_minmax<QL>(mn, mx, ql);
-        const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
-        if (FULL || off < n) {
-            if ((lane & (ql - 1)) == 0) {
-                const uint32_t qb = (uint32_t)(e0 >> q_shift) + ((uint32_t)off >> q_shift);
-                D.mn[qb] = (uint16_t)mnb;
-                D.mx[qb] = (uint16_t)mxb;
-            }
-            const float mnf = bf2f(mnb), mxf = bf2f(mxb);
-            const float u = div15(mxf - mnf, d15);
-            const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
-            const float lim = 32.0f * u;
-            float y[8];
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float x[8];
+            float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                y[e] = x[e] - mnf;
-                // fp32 data may leave the bf16-rounded range; anything beyond +-32 u clamps
-                // to an end code either way
-                if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
+                x[e] = r.val(c, e);
+                if (FULL || off + e < n) {
+                    mn = fmin_raw(mn, x[e]);
+                    mx = fmax_raw(mx, x[e]);
+                }
             }
-            bool ok = true;
-            float us = u;
-            if (ex - 32u > 190u) {
-                // zero / non-finite range: code 0.  Otherwise bring the divisor into the
-                // exponent range where div_shared is exact by an exact power-of-two scaling
-                // of divisor and numerators; the quotient does not change.
-                ok = u != 0.0f && isfinite(u);
-                const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
-                us = ok ? u * sc : 1.0f;
+            group_minmax<QL>(mn, mx, ql);
+            const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
+            if (FULL || off < n) {
+                if ((lane & (ql - 1)) == 0) {
+                    const unsigned qb = (unsigned)off >> q_shift;
+                    mnp[qb] = (uint16_t)mnb;
+                    mxp[qb] = (uint16_t)mxb;
+                }
+                const float mnf = bf2f(mnb), mxf = bf2f(mxb);
+                const float u = div15(mxf - mnf, d15);
+                const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
+                const float lim = 32.0f * u;
+                float y[8];
 #pragma unroll
-                for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
-            }
-            const Divisor dv = make_divisor(us);
-            // codes gathered as small exact floats: two 16-bit halves, nibble order
-            // (e0 e1)(e2 e3) | (e4 e5)(e6 e7) with the even element in the high nibble
-            float cf[8];
+                for (int e = 0; e < kChunk; ++e) {
+                    y[e] = x[e] - mnf;
+                    // fp32 data may leave the bf16-rounded range; anything beyond +-32 u
+                    // clamps to an end code either way
+                    if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
+                }
+                bool ok = true;
+                float us = u;
+                if (ex - 32u > 190u) {
+                    // zero / non-finite range: code 0.  Otherwise bring the divisor into the
+                    // exponent range where div_shared is exact by an exact power-of-two
+                    // scaling of divisor and numerators; the quotient does not change.
+                    ok = u != 0.0f && isfinite(u);
+                    const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
+                    us = ok ? u * sc : 1.0f;
 #pragma unroll
-            for (int e = 0; e < kChunk; ++e) {
-                float v = div_shared(y[e], dv);
-                v = floorf(v + 0.5f);
-                if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
-                cf[e] = (FULL || off + e < n) ? v : 0.0f;
+                    for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
+                }
+                const Divisor dv = make_divisor(us);
+                // codes gathered as small exact floats: two 16-bit halves, nibble order
+                // (e0 e1)(e2 e3) | (e4 e5)(e6 e7) with the even element in the high nibble
+                float cf[8];
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    float v = div_shared(y[e], dv);
+                    v = floorf(v + 0.5f);
+                    if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+                    cf[e] = (FULL || off + e < n) ? v : 0.0f;
+                }
+                float lo = cf[2];
+                lo = __builtin_fmaf(lo, 16.0f, cf[3]);
+                lo = __builtin_fmaf(lo, 16.0f, cf[0]);
+                lo = __builtin_fmaf(lo, 16.0f, cf[1]);
+                float hi = cf[6];
+                hi = __builtin_fmaf(hi, 16.0f, cf[7]);
+                hi = __builtin_fmaf(hi, 16.0f, cf[4]);
+                hi = __builtin_fmaf(hi, 16.0f, cf[5]);
+                uint32_t codes = (uint32_t)lo | ((uint32_t)hi << 16);
+                codes = ok ? codes : 0u;
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
             }
-            float lo = cf[2];
-            lo = __builtin_fmaf(lo, 16.0f, cf[3]);
-            lo = __builtin_fmaf(lo, 16.0f, cf[0]);
-            lo = __builtin_fmaf(lo, 16.0f, cf[1]);
-            float hi = cf[6];
-            hi = __builtin_fmaf(hi, 16.0f, cf[7]);
-            hi = __builtin_fmaf(hi, 16.0f, cf[4]);
-            hi = __builtin_fmaf(hi, 16.0f, cf[5]);
-            uint32_t cw = (uint32_t)lo | ((uint32_t)hi << 16);
-            cw = ok ? cw : 0u;
-            if (FULL || off + kChunk <= n) {
-                *reinterpret_cast<uint32_t *>(err + (off >> 1)) = cw;
-            } else {
-                const int nbytes = (n - off + 1) >> 1;
-                for (int j = 0; j < nbytes; ++j) err[(off >> 1) + j] = (uint8_t)(cw >> (8 * j));
-            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
+        pt.mark(11);
     }
-    pt.mark(11);
 
-    // ---- Adam direction from the window (MA:277-291); the slot cells end up holding the
-    //      update's bits, 0 where no window row names the coordinate
-    __syncthreads();  // the histogram's LDS is reused below
-    for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
-        reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
-    if (fast_window) {
-        // One entry per thread and row.  Entry (row, tid) owns row*kb + tid of z1 / z2 / coord;
-        // the first entry (in row order) to name a coordinate becomes its owner and later
-        // rows add into the owner's sums.  Rows are separated by barriers and a row never
-        // names a coordinate twice, so the sums are formed in row order.
-        __syncthreads();
-        pt.mark(12);
+    // ---- Adam direction from the window (MA:277-291), then p = p * (1 - lr*wd) (MA:234-235)
+    //      and p += -lr * u (MA:304).  The slot cells end up holding the update's bits, 0
+    //      where no window row names the coordinate.
+    __device__ __forceinline__ void update(const BlockGeo &G) {
+        const int n = FULL ? C * 2048 : G.n;
+        const int kb = G.kb;
+        const int rows = P.W.rows;
+        const TensorDesc &D = G.D;
+        __syncthreads();  // the LDS of the selection is reused below
+        for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
+            reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+        if (fast_window(G)) {
+            // One entry per thread and row.  Entry (row, tid) owns row*kb + tid of z1 / z2 /
+            // coord; the first entry (in row order) to name a coordinate becomes its owner
+            // and later rows add into the owner's sums.  Rows are separated by barriers and a
+            // row never names a coordinate twice, so the sums are formed in row order.
+            __syncthreads();
+            pt.mark(12);
 #pragma unroll
-        for (int row = 0; row < kPrefetchRows; ++row) {
-            if (row < rows) {
-                uint32_t en = ent[row];
-                if (row == D.row && tid < kb)
-                    en = (uint32_t)sel_idx[tid] | ((uint32_t)sel_val[tid] << 16);
-                const int idx = (int)(en & 0xffffu);
-                const uint32_t vb = en >> 16;
-                // +-0 values add nothing and are skipped (the rows of a fresh window are all
-                // (index 0, value 0)); idx < n also keeps a corrupt index inside the block
-                const bool active = tid < kb && idx < n && (vb & 0x7fffu) != 0;
-                const int own = row * kb + tid;
-                if (tid < kb) {
-                    const float v = bf2f(vb);
-                    const float a1 = P.W.w1[row] * v;
-                    const float vv = v * v;
-                    const float a2 = P.W.w2[row] * vv;
-                    uint32_t owner_idx = 0xffffu;
-                    if (active) {
-                        const uint32_t s = slot[idx];
-                        if (s == 0) {
-                            slot[idx] = (slot_t)(own + 1);
-                            z1[own] = 0.0f + a1;
-                            z2[own] = 0.0f + a2;
-                            owner_idx = (uint32_t)idx;
-                        } else {
-                            z1[s - 1] = z1[s - 1] + a1;
-                            z2[s - 1] = z2[s - 1] + a2;
-                        }
+            for (int row = 0; row < kPrefetchRows; ++row) {
+                if (row < rows) {
+                    int idx = (int)entI[row];
+                    uint32_t vb = entV[row];
+                    if (row == D.row && tid < kb) {
+                        idx = sel_idx[tid];
+                        vb = sel_val[tid];
                     }
-                    coord[own] = (uint16_t)owner_idx;
+                    // +-0 values add nothing and are skipped (the rows of a fresh window are
+                    // all (index 0, value 0)); idx < n also keeps a corrupt index inside
+                    const bool active = tid < kb && idx < n && (vb & 0x7fffu) != 0;
+                    const int own = row * kb + tid;
+                    if (tid < kb) {
+                        const float v = bf2f(vb);
+                        const float a1 = P.W.w1[row] * v;
+                        const float vv = v * v;
+                        const float a2 = P.W.w2[row] * vv;
+                        uint32_t owner_idx = 0xffffu;
+                        if (active) {
+                            const uint32_t s = slot[idx];
+                            if (s == 0) {
+                                slot[idx] = (slot_t)(own + 1);
+                                z1[own] = 0.0f + a1;
+                                z2[own] = 0.0f + a2;
+                                owner_idx = (uint32_t)idx;
+                            } else {
+                                z1[s - 1] = z1[s - 1] + a1;
+                                z2[s - 1] = z2[s - 1] + a2;
+                            }
+                        }
+                        coord[own] = (uint16_t)owner_idx;
+                    }
+                    __syncthreads();
+                }
+            }
+            pt.mark(13);
+            const int entries = rows * kb;
+            for (int s = tid; s < entries; s += kWG) {
+                const uint32_t ci = coord[s];
+                if (ci != 0xffffu) {
+                    const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
+                    slot[ci] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                }
+            }
+            __syncthreads();
+            pt.mark(14);
+        } else {
+            WindowView wv;
+            wv.I = D.I + G.col0;
+            wv.V = D.V + G.col0;
+            wv.k = D.k;
+            wv.rows = rows;
+            wv.cur_row = D.row;
+            wv.cur_idx = sel_idx;
+            wv.cur_val = sel_val;
+            wv.w1 = P.W.w1;
+            wv.w2 = P.W.w2;
+            for (int lo = 0; lo < n; lo += P.L.sub_len) {
+                const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+                window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
+                const int cnt =
+                    (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
+                for (int s = tid; s < cnt; s += kWG) {
+                    const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
+                    slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
                 }
                 __syncthreads();
             }
         }
-        pt.mark(13);
-        const int entries = rows * kb;
-        for (int s = tid; s < entries; s += kWG) {
-            const uint32_t ci = coord[s];
-            if (ci != 0xffffu) {
-                const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
-                slot[ci] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
-            }
-        }
-        __syncthreads();
-        pt.mark(14);
-    } else {
-        WindowView wv;
-        wv.I = D.I + col0;
-        wv.V = D.V + col0;
-        wv.k = D.k;
-        wv.rows = rows;
-        wv.cur_row = D.row;
-        wv.cur_idx = sel_idx;
-        wv.cur_val = sel_val;
-        wv.w1 = P.W.w1;
-        wv.w2 = P.W.w2;
-        for (int lo = 0; lo < n; lo += P.L.sub_len) {
-            const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
-            window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
-            const int cnt =
-                (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
-            for (int s = tid; s < cnt; s += kWG) {
-                const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
-                slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
-            }
-            __syncthreads();
-        }
-    }
-    pt.mark(15);
+        pt.mark(15);
 
-    // ---- p = p * (1 - lr*wd) (MA:234-235); p += -lr * u (MA:304)
-    const float neg_lr = D.neg_lr, decay = D.decay;
-    const bool apply_decay = D.apply_decay != 0;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-        const int off = chunk_off<C>(wave, c, lane);
-        if (FULL || off < n) {
-            float pv[8], uv[8];
-            praw[c].to_float(pv);
-            if (R::kBF16) {
-                const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
-                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                if (R::kBF16) {
+                    const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
+                    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    uv[2 * i] = __uint_as_float(w[i] << 16);
-                    uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                    for (int i = 0; i < 4; ++i) {
+                        uv[2 * i] = __uint_as_float(w[i] << 16);
+                        uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                    }
+                } else {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
+                    const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
+                    uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
+                    uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
+                    uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
+                    uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
                 }
-            } else {
-                const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
-                const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
-                uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
-                uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
-                uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
-                uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
-            }
-            if (apply_decay) {
+                if (apply_decay) {
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        pv[e] = pv[e] * decay;
+                        if (R::kBF16) pv[e] = bf2f(f2bf(pv[e]));
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
-                    pv[e] = pv[e] * decay;
-                    if (R::kBF16) pv[e] = bf2f(f2bf(pv[e]));
+                    const float prod = neg_lr * uv[e];
+                    pv[e] = pv[e] + prod;
                 }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
-#pragma unroll
-            for (int e = 0; e < kChunk; ++e) {
-                const float prod = neg_lr * uv[e];
-                pv[e] = pv[e] + prod;
-            }
-            store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
+        pt.mark(16);
     }
-    pt.mark(16);
+};
+
+// which tensor owns workgroup / work item `w` of the launch (first_block is ascending)
+__device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
+    int ti = 0;
+    for (int i = 1; i < P.n_tensors; ++i)
+        if (w >= P.t[i].first_block) ti = i;
+    return ti;
 }
 
-// QL: lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any q.
+// One workgroup per block: any block shape.  Tensor i contributes its blocks
+// blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
 template <class R, int MIN_WAVES, int QL>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
-#ifdef MA_STAGGER
-    // Workgroups that start together stay in step (same work, same duration), so the
-    // memory-bound and compute-bound phases of all workgroups on the chip coincide.  The
-    // first generation breaks the step: the workgroup in the odd wave slot of each SIMD waits
-    // about half a block time before it starts.
-    if (blockIdx.x < (unsigned)MA_STAGGER_FIRST) {
-        const unsigned hw = __builtin_amdgcn_s_getreg((3 << 11) | 4);  // HW_ID[3:0] = wave slot
-        if (hw & 1u) {
-            for (int i = 0; i < MA_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
-        }
+    const int ti = find_tensor(P, (int)blockIdx.x);
+    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
+    if (G.n == R::kC * 2048) {
+        FusedBlock<R, true, QL> fb(P, lds);
+        fb.load_params_window(G);
+        fb.load_grad_inputs(G);
+        fb.dequant(G);
+        fb.topk_and_row(G);
+        fb.quantize(G);
+        fb.update(G);
+    } else {
+        FusedBlock<R, false, QL> fb(P, lds);
+        fb.load_params_window(G);
+        fb.load_grad_inputs(G);
+        fb.dequant(G);
+        fb.topk_and_row(G);
+        fb.quantize(G);
+        fb.update(G);
     }
-#endif
-    // which tensor, which block
-    int ti = 0;
-    for (int i = 1; i < P.n_tensors; ++i)
-        if ((int)blockIdx.x >= P.t[i].first_block) ti = i;
-    const TensorDesc &D = P.t[ti];
-    const int64_t b = (int)blockIdx.x - D.first_block;
-    const int64_t dbs = D.d < P.d_block_size ? D.d : P.d_block_size;
-    const int64_t left = D.d - b * dbs;
-#ifdef MA_ANALYZE_FULL_ONLY  // development aid: a listing with the full-block path alone
-    fused_block<R, true, QL>(P, D, b, lds);
-#else
-    if (dbs == R::kC * 2048 && left >= dbs)
-        fused_block<R, true, QL>(P, D, b, lds);
-    else
-        fused_block<R, false, QL>(P, D, b, lds);
-#endif
+}
+
+// Persistent workgroups over full blocks only (every work item is a block of exactly 2048*C
+// elements; tensor i contributes its blocks 0 .. count-1).  The parameters and window rows of
+// a block are requested when its selection starts, and the next block's gradient and error
+// feedback while the current block is updated, so the workgroup has loads in flight during
+// nearly all of its arithmetic.
+template <class R, int MIN_WAVES, int QL>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_persistent(FusedParams P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int total = P.total_items;
+    int item = (int)blockIdx.x;
+    if (item >= total) return;
+    FusedBlock<R, true, QL> fb(P, lds);
+    int ti = find_tensor(P, item);
+    BlockGeo G = make_geo(P, ti, item - P.t[ti].first_block);
+    fb.load_grad_inputs(G);
+    for (;;) {
+        // the lane's offsets are rebuilt from an opaque thread id in every round: hoisted out
+        // of this loop they would tie up a hundred registers for its whole duration
+        fb.tid = opaque_tid();
+        fb.lane = fb.tid & 63;
+        fb.wave = fb.tid >> 6;
+        fb.dequant(G);
+        fb.load_params_window(G);  // arrives during the selection and quantisation
+        fb.topk_and_row(G);
+        fb.quantize(G);
+        const int next = item + (int)gridDim.x;
+        const bool more = next < total;
+        BlockGeo N = G;
+        if (more) {
+            ti = find_tensor(P, next);
+            N = make_geo(P, ti, next - P.t[ti].first_block);
+            fb.load_grad_inputs(N);  // arrives during the update of the current block
+        }
+        fb.update(G);
+        if (!more) break;
+        __syncthreads();  // the update's LDS is read to the end before the next selection
+        G = N;
+        item = next;
+    }
 }
 
 // =============================================================================================
@@ -881,6 +989,36 @@ static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, cons
     }
     return MA_ERR_BLOCK_SIZE;
 }
+
+// Persistent launch over full blocks of the hardware block size (2048 * 10 elements): as many
+// workgroups as the device keeps resident, each walking the work items with that stride.
+template <class R, int QL>
+static int launch_persistent_one(int64_t items, int lds_bytes, hipStream_t s,
+                                 const FusedParams &P) {
+    int rc = allow_big_lds(fused_step_persistent<R, 2, QL>, lds_bytes);
+    if (rc) return rc;
+    int per_cu = 0;
+    rc = (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(
+        &per_cu, reinterpret_cast<const void *>(fused_step_persistent<R, 2, QL>), kWG,
+        (size_t)lds_bytes);
+    if (rc) return rc;
+    if (per_cu < 1) per_cu = 1;
+    const int cus = ma_get_sm_count();
+    if (cus <= 0) return (int)hipErrorNoDevice;
+    int64_t grid = (int64_t)cus * per_cu;
+    if (grid > items) grid = items;
+    fused_step_persistent<R, 2, QL><<<(unsigned)grid, kWG, lds_bytes, s>>>(P);
+    return launch_status();
+}
+
+template <template <int> class RT>
+static int launch_persistent(int64_t items, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    if (P.q_shift == 6) return launch_persistent_one<RT<10>, 8>(items, lds_bytes, s, P);
+    if (P.q_shift == 5) return launch_persistent_one<RT<10>, 4>(items, lds_bytes, s, P);
+    return launch_persistent_one<RT<10>, 0>(items, lds_bytes, s, P);
+}
+
+constexpr int kPersistentChunks = 10;  // the persistent kernel exists for 20480-element bf16 blocks
 
 // geometry of one tensor, micro_adam.py:77-82
 struct Geometry {
@@ -1127,39 +1265,58 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
     window_weights(h->t, h->m, h->beta1, h->beta2, h->eps, &W);
     const int slot_bytes = h->dtype == MA_BF16 ? 2 : 4;
 
-    // launches are formed per register-tile size so that small tensors do not run in the
-    // largest kernel; inside a class, tensors go kTensorsPerLaunch at a time by value
-    static const int classes[4] = {2, 5, 10, 16};
-    for (int ci = 0; ci < 4; ++ci) {
+    // Work is handed out in launches of at most kTensorsPerLaunch tensors (their descriptors
+    // travel by value).  Full blocks of the hardware block size go to the persistent,
+    // pipelined kernel; every other block (tails, short tensors, other block sizes) goes to
+    // the one-workgroup-per-block kernel of its register-tile class.
+    const int d_block_size =
+        (int)(h->d_block_size > MA_MAX_D_BLOCK ? MA_MAX_D_BLOCK : h->d_block_size);
+    static const int classes[5] = {0, 2, 5, 10, 16};  // 0: the persistent pass
+    for (int ci = 0; ci < 5; ++ci) {
         const int C = classes[ci];
+        const bool persistent = C == 0;
         FusedParams P;
         int count = 0;
-        int64_t blocks = 0;
+        int64_t items = 0;
         int dbs_max = 0, kb_max = 0;
         auto flush = [&]() -> int {
             if (count == 0) return 0;
             P.n_tensors = count;
             P.W = W;
             P.L = plan_lds(dbs_max, kb_max, h->m, slot_bytes);
-            P.d_block_size = (int)(h->d_block_size > MA_MAX_D_BLOCK ? MA_MAX_D_BLOCK
-                                                                     : h->d_block_size);
+            P.d_block_size = d_block_size;
             P.q_shift = q_shift;
-            P.pad = 0;
+            P.total_items = (int32_t)items;
             if (P.L.total > kLdsLimit) return MA_ERR_LDS;
-            const int rc = h->dtype == MA_BF16
-                               ? launch_fused<RegsBF16>(C, (unsigned)blocks, P.L.total, s, P)
-                               : launch_fused<RegsF32>(C, (unsigned)blocks, P.L.total, s, P);
+            int rc;
+            if (persistent)
+                rc = launch_persistent<RegsBF16>(items, P.L.total, s, P);
+            else
+                rc = h->dtype == MA_BF16
+                         ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
+                         : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
             count = 0;
-            blocks = 0;
+            items = 0;
             dbs_max = kb_max = 0;
             return rc;
         };
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
             const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
-            if (chunks_for(g.dbs) != C) continue;
-            const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
-            if (count == kTensorsPerLaunch || blocks + nb > 0x7fffffff) {
+            const bool piped = h->dtype == MA_BF16 && g.dbs == 2048 * kPersistentChunks &&
+                               g.n_full > 0 && t.d >= g.dbs;
+            int64_t blk0, nb;
+            if (persistent) {
+                if (!piped) continue;
+                blk0 = 0;
+                nb = g.n_full;
+            } else {
+                if (chunks_for(g.dbs) != C) continue;
+                blk0 = piped ? g.n_full : 0;
+                nb = g.n_full + (g.tail > 0 ? 1 : 0) - blk0;
+                if (nb == 0) continue;
+            }
+            if (count == kTensorsPerLaunch || items + nb > 0x7fffffff) {
                 const int rc = flush();
                 if (rc) return rc;
             }
@@ -1176,12 +1333,12 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
             D.row = t.index;
             D.k_many = (int32_t)g.k_many;
             D.k_few = (int32_t)g.k_few;
-            D.first_block = (int32_t)blocks;
+            D.first_block = (int32_t)items;
             D.neg_lr = (float)(-t.lr);
             D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
-            D.pad = 0;
-            blocks += nb;
+            D.blk0 = (int32_t)blk0;
+            items += nb;
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
             ++count;
