@@ -22,6 +22,11 @@ sys.path.insert(0, os.path.join(ROOT, "ista-daslab-optimizers_amd"))
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
+# counters read for a plain copy of known size; (workload, op_by_op) -> bytes.  The figures and
+# the commands behind them are in profiles/.
+MEASURED_TRAFFIC = {("llama2-7b", False): 51.9e9}  # profiles/fused_step_llama2-7b_hbm_traffic.txt
+
 
 def llama2_7b():
     shapes = [(32000, 4096)]
@@ -141,6 +146,9 @@ def main():
     ap.add_argument("--grad-sets", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--op-by-op", action="store_true", help="time the unfused route instead")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB -> 1 GiB device copy, as the known-size kernel "
+                         "the FETCH_SIZE / WRITE_SIZE counters are scaled against")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -181,6 +189,12 @@ def main():
     for i in range(args.warmup):
         one_step(i)
     torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 2^30 bytes, writes 2^30 bytes
+        torch.cuda.synchronize()
+        del src, dst
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
     t0 = time.perf_counter()
@@ -209,14 +223,16 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": dtype,
+        "dtype": "f32",  # arithmetic type; storage type of p and g is config.storage
         "data": "synthetic",
-        "config": {"workload": args.workload, "params": n_params, "tensors": len(shapes), "m": m,
+        "config": {"workload": args.workload, "storage": dtype, "params": n_params,
+                   "tensors": len(shapes), "m": m,
                    "k_init": k_init, "quant_block_size": q, "alpha": alpha,
                    "d_block_size": opt.d_block_size,
                    "route": "op-by-op" if args.op_by_op else "fused"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op)),
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},
     }
