@@ -1,0 +1,61 @@
+"""Writes tests/golden/microadam_small.npz: inputs and expected outputs of a few small MicroAdam
+runs, produced by the CPU oracle (oracle/microadam_oracle.c).
+
+The reference holds no golden vectors for this path and its kernels cannot run here, so these
+fixtures record the oracle's own answers once its pins (tests/test_oracle_pins.py) are green.
+They guard the oracle against silent change and give the GPU tests inputs that do not depend
+on a random-number generator's implementation.  Run from the repository root:
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "..", "..", "oracle"))
+import microadam_oracle as oracle  # noqa: E402
+
+CASES = {
+    # name: (sizes, dtype, m, q, k_init, alpha, wd, d_block_size, steps)
+    "bf16_q64": ([3000, 257, 1024], "bf16", 4, 64, 0.01, 0.0, 0.0, 1024, 6),
+    "f32_q64_wd": ([4096], "f32", 3, 64, 0.02, 0.0, 0.01, 2048, 5),
+    "bf16_alpha": ([2500, 33], "bf16", 3, 1000, 0.01, 0.5, 0.0, 1024, 5),
+    "bf16_block20480": ([20480 + 4096], "bf16", 3, 64, 0.01, 0.0, 0.0, 20480, 4),
+}
+
+
+def main():
+    out = {}
+    rng = np.random.default_rng(20240613)
+    for name, (sizes, dtype, m, q, k_init, alpha, wd, DB, steps) in CASES.items():
+        def draw(n, std):
+            x = (rng.standard_normal(n) * std).astype(np.float32)
+            return oracle.f32_to_bf16(x) if dtype == "bf16" else x
+        params = [draw(n, 0.02) for n in sizes]
+        grads = [[draw(n, 0.01) for n in sizes] for _ in range(steps)]
+        grads[1][0][:] = 0  # one all-zero gradient: ties everywhere
+        for i, p in enumerate(params):
+            out[f"{name}/p0/{i}"] = p.copy()
+        opt = oracle.OracleMicroAdam(params, m, 1e-3, q, k_init, alpha, weight_decay=wd,
+                                     d_block_size=DB)
+        for s in range(steps):
+            for i, g in enumerate(grads[s]):
+                out[f"{name}/g/{s}/{i}"] = g.copy()
+            opt.step([g.copy() for g in grads[s]])
+        for i, p in enumerate(params):
+            st = opt.state[i]
+            I, V = oracle.canonical_window(st["I"], st["V"], st["k_block_size_many"])
+            out[f"{name}/p/{i}"] = p.copy()
+            out[f"{name}/I/{i}"] = I
+            out[f"{name}/V/{i}"] = V
+            out[f"{name}/error/{i}"] = st["error"].copy()
+            out[f"{name}/min_vals/{i}"] = st["min_vals"].copy()
+            out[f"{name}/max_vals/{i}"] = st["max_vals"].copy()
+            out[f"{name}/index/{i}"] = np.int64(st["index"])
+    np.savez_compressed(os.path.join(HERE, "microadam_small.npz"), **out)
+    print("wrote", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

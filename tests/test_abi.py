@@ -1,0 +1,75 @@
+"""The C-ABI library loads and exports every symbol include/microadam_hip.h declares; the host
+helpers mirror the reference's; without a GPU the optimizer refuses to run instead of falling
+back to anything.  No compute calls here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "microadam_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ma_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from ista_daslab_optimizers import _hip
+    names = _declared()
+    assert len(names) >= 13
+    lib = ctypes.CDLL(_hip.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(_hip.EXPORTS) == set(names)
+    assert _hip.lib.ma_get_max_floats_for_shared_memory_per_thread_block() == 40960
+    assert "window" in _hip.error_string(-3)
+
+
+def test_struct_layouts_match_header():
+    from ista_daslab_optimizers import _hip
+    # struct ma_tensor: 7 pointers, 2 int64, 2 double, 2 int32; struct ma_hyper: see header
+    assert ctypes.sizeof(_hip.MaTensor) == 7 * 8 + 2 * 8 + 2 * 8 + 2 * 4
+    assert ctypes.sizeof(_hip.MaHyper) == 8 + 4 + 4 + 8 + 8 + 4 * 8
+    assert _hip.MaTensor.lr.offset == 72 and _hip.MaTensor.index.offset == 88
+
+
+def test_host_helpers_mirror_reference():
+    from ista_daslab_optimizers.tools import CopyDirection, block_split
+    assert (CopyDirection.k2d.value, CopyDirection.d2k.value) == (0, 1)
+    assert block_split(5, 10) == (1, 5)
+    assert block_split(16777216, 20480) == (819, 16773120)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
+def test_no_gpu_is_an_error_not_a_fallback():
+    from ista_daslab_optimizers import MicroAdam
+    p = torch.nn.Parameter(torch.zeros(128))
+    with pytest.raises(RuntimeError):
+        MicroAdam([p], m=3, lr=1e-3, quant_block_size=64)
+
+
+def test_fused_step_check_rejects_bad_layouts():
+    """Host-only validation of ma_fused_step's conditions (nothing is launched)."""
+    from ista_daslab_optimizers import _hip
+    t = _hip.MaTensor()
+    for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
+        setattr(t, f, 0x10000)
+    t.d, t.k, t.lr, t.weight_decay, t.index = 20480 * 2 + 4096, 205 * 2 + 41, 1e-3, 0.0, 0
+    h = _hip.MaHyper(1, 10, _hip.MA_BF16, 64, 20480, 0.01, 0.9, 0.999, 1e-8)
+    chk = lambda: _hip.lib.ma_fused_step_check(ctypes.byref(t), ctypes.byref(h))
+    assert chk() == 0
+    t.k += 1
+    assert chk() == -4  # geometry
+    t.k -= 1
+    h.quant_block_size = 100000
+    assert chk() == _hip.MA_ERR_NOT_FUSABLE
+    h.quant_block_size = 64
+    t.g = 0x10002
+    assert chk() == _hip.MA_ERR_NOT_FUSABLE
+    t.g = 0x10000
+    h.m = 65
+    assert chk() == -3

@@ -1,0 +1,118 @@
+"""Full-size checks on the GPU, at the tensor shapes of the Llama-2-7B and outlier-1.3B lists,
+through properties that do not need the CPU oracle at that size:
+
+  * the fused kernel and the op-by-op kernels (two independent implementations of selection,
+    statistics, quantisation and update) end in bit-identical parameters and state;
+  * every block row of the window holds distinct in-range indices, and what it holds really is
+    the top-k: no unselected magnitude exceeds the smallest selected one;
+  * error feedback round trip: Qinv(e_new) reproduces the residual within half a step;
+  * parameters move only at coordinates the window names.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _canon(I, V, k_many):
+    blk = torch.arange(I.shape[1], device=I.device) // k_many
+    key = blk[None, :].long() * 65536 + I.long()
+    order = torch.argsort(key, dim=1, stable=True)
+    return torch.gather(I, 1, order), torch.gather(V.view(torch.int16), 1, order)
+
+
+def _grads(shape, kind, step, dtype):
+    g = torch.Generator(device="cuda").manual_seed(1000 + step)
+    if kind == "normal":
+        return (torch.randn(shape, generator=g, device="cuda") * 1e-3).to(dtype)
+    # Student-t(3) scaled by 1e-3 with 1 % outlier rows x100 (the stress recipe)
+    z = torch.randn(shape, generator=g, device="cuda")
+    chi = (torch.randn((3,) + tuple(shape), generator=g, device="cuda") ** 2).sum(0) / 3
+    t = z / chi.sqrt() * 1e-3
+    if len(shape) == 2:
+        rows = torch.rand(shape[0], generator=torch.Generator(device="cuda").manual_seed(7),
+                          device="cuda") < 0.01
+        t[rows] *= 100
+    return t.to(dtype)
+
+
+CASES = [
+    # shapes, m, k_init, q, grad kind, steps
+    ([(32000, 4096), (11008, 4096), (4096, 4096), (4096,)], 10, 0.01, 64, "normal", 12),
+    ([(50304, 2048), (2048, 8192)], 20, 0.05, 32, "outlier", 4),
+]
+
+
+@pytest.mark.parametrize("shapes,m,k_init,q,kind,steps", CASES)
+def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, steps):
+    from ista_daslab_optimizers import MicroAdam
+    import ista_daslab_cuda_micro_adam as ext
+    dtype = torch.bfloat16
+    torch.manual_seed(0)
+    pa = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in shapes]
+    pb = [torch.nn.Parameter(p.detach().clone()) for p in pa]
+    oa = MicroAdam(pa, m=m, lr=1e-3, quant_block_size=q, k_init=k_init)
+    ob = MicroAdam(pb, m=m, lr=1e-3, quant_block_size=q, k_init=k_init)
+    ob.use_fused = False
+    for step in range(steps):
+        grads = [_grads(s, kind, step * 10 + i, dtype) for i, s in enumerate(shapes)]
+        before = [p.detach().clone() for p in pa]
+        # accumulator a = g + Qinv(e_prev), from the op-by-op kernel
+        acc = []
+        for p, g in zip(pa, grads):
+            st = oa.state.get(p, {})
+            a = g.detach().clone().view(-1)
+            if len(st):
+                ext.asymm_block_quant_inv(a.numel(), q, st["error"], st["min_vals"], st["max_vals"], a, 1.0)
+            acc.append(a)
+        for p, g in zip(pa, grads):
+            p.grad = g.clone()
+        for p, g in zip(pb, grads):
+            p.grad = g.clone()
+        oa.step()
+        ob.step()
+        for p, p2, a, p0 in zip(pa, pb, acc, before):
+            sa, sb = oa.state[p], ob.state[p2]
+            assert oa._fusable(p, sa)
+            assert torch.equal(p.data, p2.data), f"step {step}: parameters differ between routes"
+            for key in ("error", "min_vals", "max_vals"):
+                assert torch.equal(sa[key], sb[key]), (step, key)
+            km, dbs, k = sa["k_block_size_many"], sa["d_block_size"], sa["k"]
+            Ia, Va = _canon(sa["I"], sa["V"], km)
+            Ib, Vb = _canon(sb["I"], sb["V"], km)
+            assert torch.equal(Ia, Ib) and torch.equal(Va, Vb), (step, "window")
+            # the row written in this step
+            row = (sa["index"] - 1) % m
+            idx = sa["I"][row].long()
+            assert int(idx.min()) >= 0
+            pos = (torch.arange(k, device="cuda") // km) * dbs + idx
+            assert int(pos.max()) < a.numel()
+            assert torch.unique(pos).numel() == k, "duplicate index in a block row"
+            mag = a.float().abs()
+            assert torch.equal(sa["V"][row], a[pos]), "window values are not a[I]"
+            sel = torch.zeros_like(mag, dtype=torch.bool)
+            sel[pos] = True
+            nblk = (a.numel() + dbs - 1) // dbs
+            pad = nblk * dbs - a.numel()
+            mag_p = torch.nn.functional.pad(mag, (0, pad), value=-1.0).view(nblk, dbs)
+            sel_p = torch.nn.functional.pad(sel, (0, pad), value=False).view(nblk, dbs)
+            smallest_kept = torch.where(sel_p, mag_p, torch.full_like(mag_p, float("inf"))).amin(1)
+            largest_left = torch.where(sel_p, torch.full_like(mag_p, -1.0), mag_p).amax(1)
+            assert bool((smallest_kept >= largest_left).all()), "a larger magnitude was left out"
+            # error feedback round trip
+            resid = a.clone()
+            resid[pos] = 0
+            deq = torch.zeros_like(a)
+            ext.asymm_block_quant_inv(a.numel(), q, sa["error"], sa["min_vals"], sa["max_vals"], deq, 1.0)
+            nq = (a.numel() + q - 1) // q
+            u = (sa["max_vals"][:nq].float() - sa["min_vals"][:nq].float()) / 15
+            u = u.repeat_interleave(q)[: a.numel()]
+            tol = u / 2 + resid.float().abs() * 2.0 ** -7 + 1e-12
+            assert bool(((deq.float() - resid.float()).abs() <= tol).all()), "EF round trip"
+            # parameters move only where the window points
+            live = min(step + 1, m)
+            touched = torch.zeros(a.numel(), dtype=torch.bool, device="cuda")
+            for r in range(live):
+                touched[(torch.arange(k, device="cuda") // km) * dbs + sa["I"][r].long()] = True
+            moved = (p.data.view(-1) != p0.view(-1))
+            assert not bool((moved & ~touched).any())
