@@ -427,7 +427,7 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], int
     return prefix;
 }
 
-constexpr int kCandPerWave = 128;  // candidate slots per wave; more than that falls back
+constexpr int kCandPerWave = 128;  // candidate slots per wave (a multiple of 16); more falls back
 
 // The fast top-k of a full bf16 block.  `park` (2048*C uint16 cells) receives the block;
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
@@ -437,7 +437,7 @@ constexpr int kCandPerWave = 128;  // candidate slots per wave; more than that f
 template <class R>
 __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uint32_t *hist,
                                                uint32_t *sh, uint16_t *sel_idx,
-                                               uint16_t *sel_val) {
+                                               uint16_t *sel_val, PhaseTimer &pt) {
     constexpr int C = R::kC;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t *cand = hist + kSmallHistWords;
@@ -449,7 +449,9 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
             make_uint4(r.w[c][0], r.w[c][1], r.w[c][2], r.w[c][3]);
         cmax[c] = chunk_max_key(r.w[c]);
     }
+    pt.mark(1);
     const uint32_t L = select_kth_key15<C>(cmax, kb, hist, sh);
+    pt.mark(2);
 
     // candidates: every element with key >= L, wave by wave into the wave's own list
     uint32_t todo = 0;
@@ -484,10 +486,11 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
             ++pos;
         }
     }
-    // pad the wave's list to a multiple of 4 with zeros (never greater than a candidate)
-    if (lane < 4 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
+    // pad the wave's list to a multiple of 16 with zeros (never greater than a candidate)
+    if (lane < 16 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
     if (lane == 0) sh[12 + wave] = filled;
     __syncthreads();
+    pt.mark(3);
     uint32_t cnts[kWaves];
     bool ok = true;
 #pragma unroll
@@ -514,11 +517,16 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
 #pragma unroll
             for (int w = 0; w < kWaves; ++w) {
                 const uint4 *seg = reinterpret_cast<const uint4 *>(cand + w * kCandPerWave);
-                const int quads = ((int)cnts[w] + 3) >> 2;
-                for (int j = 0; j < quads; ++j) {
-                    const uint4 o = seg[j];
-                    rank += (o.x > my ? 1u : 0u) + (o.y > my ? 1u : 0u) + (o.z > my ? 1u : 0u) +
-                            (o.w > my ? 1u : 0u);
+                const int groups = ((int)cnts[w] + 15) >> 4;  // 16 candidates per round
+                for (int j = 0; j < groups; ++j) {
+                    const uint4 o0 = seg[4 * j], o1 = seg[4 * j + 1], o2 = seg[4 * j + 2],
+                                o3 = seg[4 * j + 3];
+                    rank += (o0.x > my ? 1u : 0u) + (o0.y > my ? 1u : 0u) + (o0.z > my ? 1u : 0u) +
+                            (o0.w > my ? 1u : 0u) + (o1.x > my ? 1u : 0u) + (o1.y > my ? 1u : 0u) +
+                            (o1.z > my ? 1u : 0u) + (o1.w > my ? 1u : 0u) + (o2.x > my ? 1u : 0u) +
+                            (o2.y > my ? 1u : 0u) + (o2.z > my ? 1u : 0u) + (o2.w > my ? 1u : 0u) +
+                            (o3.x > my ? 1u : 0u) + (o3.y > my ? 1u : 0u) + (o3.z > my ? 1u : 0u) +
+                            (o3.w > my ? 1u : 0u);
                 }
             }
             if (have && rank < (uint32_t)kb) {
@@ -530,6 +538,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         }
         __syncthreads();
     }
+    pt.mark(4);
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         const int off = chunk_off<C>(wave, c, lane);

@@ -450,7 +450,14 @@ struct FusedBlock {
     uint32_t entI[kPrefetchRows];  // older window rows, kept as loaded so that nothing waits
     uint32_t entV[kPrefetchRows];  // for them before use     load_params_window -> update
     RawChunk<R> graw[C];          // gradient                load_grad_inputs   -> dequant
-    uint32_t cw[C], smn[C], smx[C];  // 4-bit codes, stats   load_grad_inputs   -> dequant
+    // 4-bit codes and statistics                            load_grad_inputs   -> dequant
+    // With a full block and a compile-time quantisation group the wave's statistics are
+    // fetched once, 64 per register (kCoStats registers per array), and handed to the lanes
+    // by cross-lane reads in dequant; otherwise every chunk loads its own pair.
+    static constexpr bool kCoop = FULL && QL > 0;
+    static constexpr int kWaveStats = kCoop ? C * kWave / (QL > 0 ? QL : 1) : 0;
+    static constexpr int kCoStats = kCoop ? (kWaveStats + kWave - 1) / kWave : 1;
+    uint32_t cw[C], smn[kCoop ? kCoStats : C], smx[kCoop ? kCoStats : C];
     R r;                          // accumulator             dequant            -> quantize
 
     __device__ __forceinline__ FusedBlock(const FusedParams &P_, unsigned char *lds) : P(P_) {
@@ -468,7 +475,9 @@ struct FusedBlock {
         wave = tid >> 6;
         q_shift = QL > 0 ? (QL == 4 ? 5 : 6) : P.q_shift;
         ql = 1 << (q_shift - 3);
-        d15 = make_divisor(15.0f);
+        // 1/15 rounded to nearest; div_shared is exact for a reciprocal within one ulp
+        d15.u = 15.0f;
+        d15.r = 0x1.111112p-4f;
         pt.begin();
     }
 
@@ -509,7 +518,12 @@ struct FusedBlock {
             const int off = chunk_off<C>(wave, c, lane);
             graw[c].load(g, off, n, FULL);
             cw[c] = 0;
-            smn[c] = smx[c] = 0;
+            if constexpr (kCoop) {
+                cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
+                continue;
+            } else {
+                smn[c] = smx[c] = 0;
+            }
             if (FULL || off < n) {
                 if (FULL || off + kChunk <= n) {
                     cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
@@ -523,6 +537,18 @@ struct FusedBlock {
                 smx[c] = mxp[qb];
             }
         }
+        if constexpr (kCoop) {
+            const unsigned wave_first = (unsigned)(wave * C * kWave) / (unsigned)QL;
+#pragma unroll
+            for (int i = 0; i < kCoStats; ++i) {
+                const unsigned j = (unsigned)(i * kWave + lane);
+                smn[i] = smx[i] = 0;
+                if (j < (unsigned)kWaveStats) {
+                    smn[i] = mnp[wave_first + j];
+                    smx[i] = mxp[wave_first + j];
+                }
+            }
+        }
     }
 
     // ---- a = g + Qinv(e), rounded to the element type (MA:190)
@@ -533,7 +559,17 @@ struct FusedBlock {
             const int off = chunk_off<C>(wave, c, lane);
             float v[8];
             graw[c].to_float(v);
-            const float mn = bf2f(smn[c]), mx = bf2f(smx[c]);
+            uint32_t mnb, mxb;
+            if constexpr (kCoop) {
+                const int j0 = c * (kWave / QL);  // first statistic of this chunk in the wave
+                const int src = (j0 & (kWave - 1)) + lane / QL;
+                mnb = (uint32_t)__shfl((int)smn[j0 >> 6], src, kWave);
+                mxb = (uint32_t)__shfl((int)smx[j0 >> 6], src, kWave);
+            } else {
+                mnb = smn[c];
+                mxb = smx[c];
+            }
+            const float mn = bf2f(mnb), mx = bf2f(mxb);
             const float u = div15(mx - mn, d15);
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
@@ -561,7 +597,7 @@ struct FusedBlock {
         if constexpr (FULL && R::kBF16) {
             if (kb <= kWG) {
                 topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
-                                           sel_idx, sel_val);
+                                           sel_idx, sel_val, pt);
                 launder(r);
                 pt.mark(7);
             }
@@ -865,17 +901,17 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_persistent(FusedPar
         fb.quantize(G);
         const int next = item + (int)gridDim.x;
         const bool more = next < total;
-        BlockGeo N = G;
         if (more) {
-            ti = find_tensor(P, next);
-            N = make_geo(P, ti, next - P.t[ti].first_block);
+            const int tn = find_tensor(P, next);
+            const BlockGeo N = make_geo(P, tn, next - P.t[tn].first_block);
             fb.load_grad_inputs(N);  // arrives during the update of the current block
         }
         fb.update(G);
         if (!more) break;
         __syncthreads();  // the update's LDS is read to the end before the next selection
-        G = N;
         item = next;
+        ti = find_tensor(P, item);
+        G = make_geo(P, ti, item - P.t[ti].first_block);
     }
 }
 
