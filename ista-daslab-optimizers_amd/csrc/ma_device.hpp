@@ -381,48 +381,70 @@ __device__ __forceinline__ uint32_t chunk_max_key(const uint32_t (&w)[4]) {
 }
 
 constexpr int kSmallCopies = 8;
-constexpr int kSmallHistWords = 257 * kSmallCopies;
+constexpr int kSmallHistWords = 2 * 257 * kSmallCopies;  // one histogram per pass
 
 // kb-th largest of the N * 256 keys (15 bits each) held N per thread; 1 <= kb <= N * 256.
-// hist: kSmallHistWords words, sh: 8 words.  Ends with a barrier.
+// Two radix passes (8 + 7 bits).  Every thread counts its keys into a replicated LDS
+// histogram; wave 0 alone then walks the 256 bins from the top (4 bins per lane, a DPP prefix
+// sum across lanes) and publishes the digit that holds the kb-th key, which costs two
+// barriers per pass instead of a workgroup-wide scan.
+//   hist: kSmallHistWords words, sh: 8 words.  Ends with a barrier.
+//   valid: bit i set if v[i] takes part.  take_eq: how many keys equal to the result belong
+//   to the top kb; n_eq: how many keys equal it in all.
 template <int N>
-__device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], int kb,
-                                                     uint32_t *hist, uint32_t *sh) {
+__device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uint32_t valid,
+                                                     int kb, uint32_t *hist, uint32_t *sh,
+                                                     int &take_eq, int &n_eq) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < kSmallHistWords / 4; i += kWG)
+        reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
     uint32_t prefix = 0, pmask = 0;
     int need = kb;
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
         const int shift = pass == 0 ? 7 : 0;
-        const int nb = pass == 0 ? 256 : 128;
-        const uint32_t dm = nb - 1;
-        for (int i = tid; i < nb * kSmallCopies / 4; i += kWG)
-            reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
-        __syncthreads();
+        const uint32_t dm = pass == 0 ? 255u : 127u;
+        uint32_t *h = hist + pass * 257 * kSmallCopies;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
-            const uint32_t bin = (v[i] & pmask) == prefix ? ((v[i] >> shift) & dm) : 256u;
-            atomicAdd(&hist[bin * kSmallCopies + (lane & (kSmallCopies - 1))], 1u);
+            const bool in = ((valid >> i) & 1u) != 0 && (v[i] & pmask) == prefix;
+            const uint32_t bin = in ? ((v[i] >> shift) & dm) : 256u;
+            atomicAdd(&h[bin * kSmallCopies + (lane & (kSmallCopies - 1))], 1u);
         }
         __syncthreads();
-        const int bin = nb - 1 - tid;
-        uint32_t cnt = 0;
-        if (bin >= 0) {
-            const uint4 a = reinterpret_cast<const uint4 *>(hist)[bin * 2];
-            const uint4 b = reinterpret_cast<const uint4 *>(hist)[bin * 2 + 1];
-            cnt = a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
-        }
-        const uint32_t incl = wg_incl_scan(cnt, sh, lane, wave);
-        const uint32_t excl = incl - cnt;
-        if (bin >= 0 && excl < (uint32_t)need && (uint32_t)need <= incl) {
-            sh[4] = (uint32_t)bin;
-            sh[5] = (uint32_t)need - excl;
+        if (wave == 0) {
+            // lane l owns bins 255-4l .. 252-4l (bins above dm are empty in the second pass)
+            uint32_t c[4], tot = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int bin = 255 - 4 * lane - i;
+                const uint4 a = reinterpret_cast<const uint4 *>(h)[bin * 2];
+                const uint4 b = reinterpret_cast<const uint4 *>(h)[bin * 2 + 1];
+                c[i] = a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
+                tot += c[i];
+            }
+            const uint32_t incl = wave_incl_scan(tot, lane);
+            uint32_t above = incl - tot;  // keys in bins above this lane's
+            if (above < (uint32_t)need && (uint32_t)need <= incl) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (above < (uint32_t)need && (uint32_t)need <= above + c[i]) {
+                        sh[4] = (uint32_t)(255 - 4 * lane - i);
+                        sh[5] = (uint32_t)need - above;
+                        sh[7] = c[i];
+                    }
+                    above += c[i];
+                }
+            }
         }
         __syncthreads();
         prefix |= sh[4] << shift;
         pmask |= dm << shift;
         need = (int)sh[5];
     }
+    take_eq = need;
+    n_eq = (int)sh[7];
     __syncthreads();
     return prefix;
 }
@@ -434,6 +456,8 @@ constexpr int kCandPerWave = 128;  // candidate slots per wave (a multiple of 16
 // magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false
 // (a wave found more candidates than it has room for: heavy ties) r is reloaded unchanged.
 //   hist: kSmallHistWords + 4*kCandPerWave words; sh: 16 words.  1 <= kb <= 256.
+// Output order: entries above the threshold key in candidate-list order, then the kept
+// entries equal to it by increasing index; deterministic for given data.
 template <class R>
 __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uint32_t *hist,
                                                uint32_t *sh, uint16_t *sel_idx,
@@ -450,7 +474,8 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         cmax[c] = chunk_max_key(r.w[c]);
     }
     pt.mark(1);
-    const uint32_t L = select_kth_key15<C>(cmax, kb, hist, sh);
+    int unused_take, unused_eq;
+    const uint32_t L = select_kth_key15<C>(cmax, 0xffffffffu, kb, hist, sh, unused_take, unused_eq);
     pt.mark(2);
 
     // candidates: every element with key >= L, wave by wave into the wave's own list
@@ -499,41 +524,68 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         ok = ok && cnts[w] <= (uint32_t)kCandPerWave;
     }
     if (ok) {
-        // rank of each candidate among all candidates: composites are distinct, larger wins
-        const int total = (int)(cnts[0] + cnts[1] + cnts[2] + cnts[3]);
-        for (int base = 0; base < total; base += kWG) {
-            int i = base + tid;
-            uint32_t my = 0;
-            bool have = false;
+        // Exact top-kb among the candidates (at most two per thread): a radix select on their
+        // keys gives the threshold key T and the number of entries equal to T to keep; entries
+        // above T get consecutive output slots by a prefix sum over the threads, entries equal
+        // to T are ranked among themselves by index (they are few).
+        uint32_t my[2] = {0, 0};
+        uint32_t have = 0;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            int i = s * kWG + tid;
+            bool got = false;
 #pragma unroll
             for (int w = 0; w < kWaves; ++w) {
-                if (!have && i >= 0 && i < (int)cnts[w]) {
-                    my = cand[w * kCandPerWave + i];
-                    have = true;
+                if (!got && i < (int)cnts[w]) {
+                    my[s] = cand[w * kCandPerWave + i];
+                    got = true;
                 }
                 i -= (int)cnts[w];
+                if (i < 0) i = 0x7fffffff;  // already placed, or in a list further on
             }
-            uint32_t rank = 0;
+            have |= (got ? 1u : 0u) << s;
+        }
+        const uint32_t keys[2] = {my[0] >> 15, my[1] >> 15};
+        if (tid == 0) sh[6] = 0;
+        int take_eq, n_eq;
+        const uint32_t T = select_kth_key15<2>(keys, have, kb, hist, sh, take_eq, n_eq);
+        uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the histogram is free again
+        constexpr int kMaxTies = 512;
+        ok = n_eq <= kMaxTies;
+        if (ok) {
+            uint32_t n_gt = 0;
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                const uint4 *seg = reinterpret_cast<const uint4 *>(cand + w * kCandPerWave);
-                const int groups = ((int)cnts[w] + 15) >> 4;  // 16 candidates per round
-                for (int j = 0; j < groups; ++j) {
-                    const uint4 o0 = seg[4 * j], o1 = seg[4 * j + 1], o2 = seg[4 * j + 2],
-                                o3 = seg[4 * j + 3];
-                    rank += (o0.x > my ? 1u : 0u) + (o0.y > my ? 1u : 0u) + (o0.z > my ? 1u : 0u) +
-                            (o0.w > my ? 1u : 0u) + (o1.x > my ? 1u : 0u) + (o1.y > my ? 1u : 0u) +
-                            (o1.z > my ? 1u : 0u) + (o1.w > my ? 1u : 0u) + (o2.x > my ? 1u : 0u) +
-                            (o2.y > my ? 1u : 0u) + (o2.z > my ? 1u : 0u) + (o2.w > my ? 1u : 0u) +
-                            (o3.x > my ? 1u : 0u) + (o3.y > my ? 1u : 0u) + (o3.z > my ? 1u : 0u) +
-                            (o3.w > my ? 1u : 0u);
+            for (int s = 0; s < 2; ++s) n_gt += (((have >> s) & 1u) != 0 && keys[s] > T) ? 1u : 0u;
+            const uint32_t incl = wg_incl_scan(n_gt, sh, lane, wave);
+            uint32_t pos = incl - n_gt;
+            uint32_t tie_idx[2] = {0xffffu, 0xffffu};
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (((have >> s) & 1u) == 0) continue;
+                const uint32_t idx = 32767u - (my[s] & 0x7fffu);
+                if (keys[s] > T) {
+                    sel_idx[pos] = (uint16_t)idx;
+                    sel_val[pos] = park[idx];
+                    park[idx] = 0;
+                    ++pos;
+                } else if (keys[s] == T) {
+                    const uint32_t at = atomicAdd(&sh[6], 1u);
+                    ties[at] = (uint16_t)idx;
+                    tie_idx[s] = idx;
                 }
             }
-            if (have && rank < (uint32_t)kb) {
-                const uint32_t idx = 32767u - (my & 0x7fffu);
-                sel_idx[rank] = (uint16_t)idx;
-                sel_val[rank] = park[idx];
-                park[idx] = 0;
+            __syncthreads();
+            const int first_eq = kb - take_eq;  // output slots before the ties
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (tie_idx[s] == 0xffffu) continue;
+                uint32_t rank = 0;
+                for (int j = 0; j < n_eq; ++j) rank += ties[j] < tie_idx[s] ? 1u : 0u;
+                if (rank < (uint32_t)take_eq) {
+                    sel_idx[first_eq + rank] = (uint16_t)tie_idx[s];
+                    sel_val[first_eq + rank] = park[tie_idx[s]];
+                    park[tie_idx[s]] = 0;
+                }
             }
         }
         __syncthreads();

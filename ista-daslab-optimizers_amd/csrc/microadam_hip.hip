@@ -594,6 +594,11 @@ struct FusedBlock {
     __device__ __forceinline__ void topk_and_row(const BlockGeo &G) {
         const int kb = G.kb;
         bool topk_done = false;
+#if defined(MA_ABLATE) && MA_ABLATE == 1  // timing experiment: no selection
+        if (tid < kb) { sel_idx[tid] = (uint16_t)tid; sel_val[tid] = 0; }
+        __syncthreads();
+        topk_done = true;
+#else
         if constexpr (FULL && R::kBF16) {
             if (kb <= kWG) {
                 topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
@@ -611,6 +616,7 @@ struct FusedBlock {
             compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
             launder(r);
         }
+#endif
         int16_t *Irow = G.D.I + ((int64_t)G.D.row * G.D.k + G.col0);
         uint16_t *Vrow = G.D.V + ((int64_t)G.D.row * G.D.k + G.col0);
         for (int j = tid; j < kb; j += kWG) {
@@ -622,6 +628,10 @@ struct FusedBlock {
 
     // ---- residual statistics (MA:217-228) and 4-bit codes (MA:231)
     __device__ __forceinline__ void quantize(const BlockGeo &G) {
+#if defined(MA_ABLATE) && MA_ABLATE == 2
+        launder(r);
+        return;
+#endif
         const int n = FULL ? C * 2048 : G.n;
         uint8_t *err = G.D.err + (G.e0 >> 1);
         uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
@@ -716,7 +726,11 @@ struct FusedBlock {
         __syncthreads();  // the LDS of the selection is reused below
         for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
             reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+#if defined(MA_ABLATE) && MA_ABLATE == 3
+        if (false) {
+#else
         if (fast_window(G)) {
+#endif
             // One entry per thread and row.  Entry (row, tid) owns row*kb + tid of z1 / z2 /
             // coord; the first entry (in row order) to name a coordinate becomes its owner
             // and later rows add into the owner's sums.  Rows are separated by barriers and a
@@ -770,7 +784,11 @@ struct FusedBlock {
             }
             __syncthreads();
             pt.mark(14);
+#if defined(MA_ABLATE) && MA_ABLATE == 3
+        } else if (false) {
+#else
         } else {
+#endif
             WindowView wv;
             wv.I = D.I + G.col0;
             wv.V = D.V + G.col0;
