@@ -12,10 +12,27 @@
 
 namespace ma {
 
-constexpr int kWG = 256;
+#ifndef MA_WG
+#define MA_WG 512  // threads per workgroup of the block kernels: 256 or 512
+#endif
+constexpr int kWG = MA_WG;
 constexpr int kWave = 64;
 constexpr int kWaves = kWG / kWave;
 constexpr int kChunk = 8;        // elements per lane per chunk
+constexpr int kRound = kWG * kChunk;  // elements one chunk of every thread covers together
+// register-tile classes: chunks per thread for blocks up to 4096 / ~10-12 K / 20480 / 32768
+constexpr int kClass0 = kWG == 256 ? 2 : 1;
+constexpr int kClass1 = kWG == 256 ? 5 : 3;
+constexpr int kClass2 = kWG == 256 ? 10 : 5;
+constexpr int kClass3 = kWG == 256 ? 16 : 8;
+// words of the small LDS scratch every block kernel has at offset 0
+constexpr int kShScan = 0;      // 8 words: per-wave partial sums
+constexpr int kShCounter = 8;   // slot allocation counter of the window pass
+constexpr int kShPivot = 9;     // radix select: digit of the pivot bin
+constexpr int kShNeed = 10;     //               keys still to take inside it
+constexpr int kShNEq = 11;      //               keys in the pivot bin
+constexpr int kShTies = 12;     // fast top-k: tie list length
+constexpr int kShCnts = 16;     // 8 words: candidates per wave
 constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
 constexpr int kMaxWindow = 64;
 
@@ -343,13 +360,13 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
         uint32_t incl = wg_incl_scan(cnt, sh, lane, wave);
         uint32_t excl = incl - cnt;
         if (bin >= 0 && excl < (uint32_t)need && (uint32_t)need <= incl) {
-            sh[4] = (uint32_t)bin;
-            sh[5] = (uint32_t)need - excl;
+            sh[kShPivot] = (uint32_t)bin;
+            sh[kShNeed] = (uint32_t)need - excl;
         }
         __syncthreads();
-        prefix |= sh[4] << shift;
+        prefix |= sh[kShPivot] << shift;
         pmask |= dm << shift;
-        need = (int)sh[5];
+        need = (int)sh[kShNeed];
         if (pass < 2) pt.mark(pt0 + 3 * pass + 2);
     }
     __syncthreads();
@@ -430,26 +447,26 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (above < (uint32_t)need && (uint32_t)need <= above + c[i]) {
-                        sh[4] = (uint32_t)(255 - 4 * lane - i);
-                        sh[5] = (uint32_t)need - above;
-                        sh[7] = c[i];
+                        sh[kShPivot] = (uint32_t)(255 - 4 * lane - i);
+                        sh[kShNeed] = (uint32_t)need - above;
+                        sh[kShNEq] = c[i];
                     }
                     above += c[i];
                 }
             }
         }
         __syncthreads();
-        prefix |= sh[4] << shift;
+        prefix |= sh[kShPivot] << shift;
         pmask |= dm << shift;
-        need = (int)sh[5];
+        need = (int)sh[kShNeed];
     }
     take_eq = need;
-    n_eq = (int)sh[7];
+    n_eq = (int)sh[kShNEq];
     __syncthreads();
     return prefix;
 }
 
-constexpr int kCandPerWave = 128;  // candidate slots per wave (a multiple of 16); more falls back
+constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multiple of 16); more falls back
 
 // The fast top-k of a full bf16 block.  `park` (2048*C uint16 cells) receives the block;
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
@@ -513,14 +530,14 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     }
     // pad the wave's list to a multiple of 16 with zeros (never greater than a candidate)
     if (lane < 16 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
-    if (lane == 0) sh[12 + wave] = filled;
+    if (lane == 0) sh[kShCnts + wave] = filled;
     __syncthreads();
     pt.mark(3);
     uint32_t cnts[kWaves];
     bool ok = true;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-        cnts[w] = sh[12 + w];
+        cnts[w] = sh[kShCnts + w];
         ok = ok && cnts[w] <= (uint32_t)kCandPerWave;
     }
     if (ok) {
@@ -528,10 +545,11 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         // keys gives the threshold key T and the number of entries equal to T to keep; entries
         // above T get consecutive output slots by a prefix sum over the threads, entries equal
         // to T are ranked among themselves by index (they are few).
+        constexpr int kMine = 512 / kWG;  // candidates per thread
         uint32_t my[2] = {0, 0};
         uint32_t have = 0;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
+        for (int s = 0; s < kMine; ++s) {
             int i = s * kWG + tid;
             bool got = false;
 #pragma unroll
@@ -546,7 +564,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
             have |= (got ? 1u : 0u) << s;
         }
         const uint32_t keys[2] = {my[0] >> 15, my[1] >> 15};
-        if (tid == 0) sh[6] = 0;
+        if (tid == 0) sh[kShTies] = 0;
         int take_eq, n_eq;
         const uint32_t T = select_kth_key15<2>(keys, have, kb, hist, sh, take_eq, n_eq);
         uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the histogram is free again
@@ -569,7 +587,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
                     park[idx] = 0;
                     ++pos;
                 } else if (keys[s] == T) {
-                    const uint32_t at = atomicAdd(&sh[6], 1u);
+                    const uint32_t at = atomicAdd(&sh[kShTies], 1u);
                     ties[at] = (uint16_t)idx;
                     tie_idx[s] = idx;
                 }

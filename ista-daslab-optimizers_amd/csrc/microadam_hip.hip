@@ -235,7 +235,7 @@ struct LdsMap {
     int sub_len;      // coordinates handled per window pass
     int total;        // bytes
 };
-constexpr int kMiscBytes = 64;  // sh[8] words + counter at the very start
+constexpr int kMiscBytes = 128;  // the kSh* words at the very start
 constexpr int kHistBytes = 257 * kHistCopies * 4;
 
 struct WindowWeights {
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kWG) void window_update_kernel(int64_t d, int dbs, 
                                                             WindowWeights W, LdsMap L) {
     extern __shared__ __align__(16) unsigned char lds[];
     uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
-    uint32_t *counter = sh + 8;
+    uint32_t *counter = sh + kShCounter;
     uint16_t *slot = reinterpret_cast<uint16_t *>(lds + L.off_slot);
     float *z1 = reinterpret_cast<float *>(lds + L.off_union);
     float *z2 = z1 + L.z_cap;
@@ -354,7 +354,7 @@ struct FusedParams {
     int32_t n_tensors;
     int32_t d_block_size;
     int32_t q_shift;  // log2(quant_block_size)
-    int32_t total_items;  // work items of the launch (persistent kernel)
+    int32_t total_items;  // work items (blocks) of the launch
 };
 
 template <class R>
@@ -426,9 +426,8 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
     return G;
 }
 
-// The step of one block, cut into stages so that a persistent workgroup can request the next
-// block's inputs while it works on the current one.  The register arrays are members; the
-// stages say which of them they fill and which they consume.
+// The step of one block, cut into stages.  The register arrays are members; the stages say
+// which of them they fill and which they consume.
 //   FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
 //   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
 template <class R, bool FULL, int QL>
@@ -462,7 +461,7 @@ struct FusedBlock {
 
     __device__ __forceinline__ FusedBlock(const FusedParams &P_, unsigned char *lds) : P(P_) {
         sh = reinterpret_cast<uint32_t *>(lds);
-        counter = sh + 8;
+        counter = sh + kShCounter;
         sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
         sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
         slot = reinterpret_cast<slot_t *>(lds + P.L.off_slot);
@@ -487,7 +486,7 @@ struct FusedBlock {
 
     // ---- parameters and the older window rows: requested early, consumed last
     __device__ __forceinline__ void load_params_window(const BlockGeo &G) {
-        const int n = FULL ? C * 2048 : G.n;
+        const int n = FULL ? C * kRound : G.n;
         const elem_t *p = reinterpret_cast<const elem_t *>(G.D.p) + G.e0;
 #pragma unroll
         for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
@@ -508,7 +507,7 @@ struct FusedBlock {
 
     // ---- gradient, 4-bit error feedback and its statistics
     __device__ __forceinline__ void load_grad_inputs(const BlockGeo &G) {
-        const int n = FULL ? C * 2048 : G.n;
+        const int n = FULL ? C * kRound : G.n;
         const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
         const uint8_t *err = G.D.err + (G.e0 >> 1);
         const uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
@@ -553,7 +552,7 @@ struct FusedBlock {
 
     // ---- a = g + Qinv(e), rounded to the element type (MA:190)
     __device__ __forceinline__ void dequant(const BlockGeo &G) {
-        const int n = FULL ? C * 2048 : G.n;
+        const int n = FULL ? C * kRound : G.n;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -632,7 +631,7 @@ struct FusedBlock {
         launder(r);
         return;
 #endif
-        const int n = FULL ? C * 2048 : G.n;
+        const int n = FULL ? C * kRound : G.n;
         uint8_t *err = G.D.err + (G.e0 >> 1);
         uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
         uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
@@ -719,7 +718,7 @@ struct FusedBlock {
     //      and p += -lr * u (MA:304).  The slot cells end up holding the update's bits, 0
     //      where no window row names the coordinate.
     __device__ __forceinline__ void update(const BlockGeo &G) {
-        const int n = FULL ? C * 2048 : G.n;
+        const int n = FULL ? C * kRound : G.n;
         const int kb = G.kb;
         const int rows = P.W.rows;
         const TensorDesc &D = G.D;
@@ -873,7 +872,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     extern __shared__ __align__(16) unsigned char lds[];
     const int ti = find_tensor(P, (int)blockIdx.x);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
-    if (G.n == R::kC * 2048) {
+    if (G.n == R::kC * kRound) {
         FusedBlock<R, true, QL> fb(P, lds);
         fb.load_params_window(G);
         fb.load_grad_inputs(G);
@@ -889,47 +888,6 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         fb.topk_and_row(G);
         fb.quantize(G);
         fb.update(G);
-    }
-}
-
-// Persistent workgroups over full blocks only (every work item is a block of exactly 2048*C
-// elements; tensor i contributes its blocks 0 .. count-1).  The parameters and window rows of
-// a block are requested when its selection starts, and the next block's gradient and error
-// feedback while the current block is updated, so the workgroup has loads in flight during
-// nearly all of its arithmetic.
-template <class R, int MIN_WAVES, int QL>
-__global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_persistent(FusedParams P) {
-    extern __shared__ __align__(16) unsigned char lds[];
-    const int total = P.total_items;
-    int item = (int)blockIdx.x;
-    if (item >= total) return;
-    FusedBlock<R, true, QL> fb(P, lds);
-    int ti = find_tensor(P, item);
-    BlockGeo G = make_geo(P, ti, item - P.t[ti].first_block);
-    fb.load_grad_inputs(G);
-    for (;;) {
-        // the lane's offsets are rebuilt from an opaque thread id in every round: hoisted out
-        // of this loop they would tie up a hundred registers for its whole duration
-        fb.tid = opaque_tid();
-        fb.lane = fb.tid & 63;
-        fb.wave = fb.tid >> 6;
-        fb.dequant(G);
-        fb.load_params_window(G);  // arrives during the selection and quantisation
-        fb.topk_and_row(G);
-        fb.quantize(G);
-        const int next = item + (int)gridDim.x;
-        const bool more = next < total;
-        if (more) {
-            const int tn = find_tensor(P, next);
-            const BlockGeo N = make_geo(P, tn, next - P.t[tn].first_block);
-            fb.load_grad_inputs(N);  // arrives during the update of the current block
-        }
-        fb.update(G);
-        if (!more) break;
-        __syncthreads();  // the update's LDS is read to the end before the next selection
-        item = next;
-        ti = find_tensor(P, item);
-        G = make_geo(P, ti, item - P.t[ti].first_block);
     }
 }
 
@@ -989,13 +947,14 @@ static int allow_big_lds(K kernel, int bytes) {
 }
 
 constexpr int kLdsLimit = 160 * 1024;
+constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
 // chunks per thread that cover a block of `dbs` elements; 0 if none does
 static int chunks_for(int64_t dbs) {
-    if (dbs <= 2048 * 2) return 2;
-    if (dbs <= 2048 * 5) return 5;
-    if (dbs <= 2048 * 10) return 10;
-    if (dbs <= 2048 * 16) return 16;
+    if (dbs <= kRound * kClass0) return kClass0;
+    if (dbs <= kRound * kClass1) return kClass1;
+    if (dbs <= kRound * kClass2) return kClass2;
+    if (dbs <= kRound * kClass3) return kClass3;
     return 0;
 }
 
@@ -1013,10 +972,10 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
         return launch_status();                                                              \
     }
     switch (C) {
-        MA_TOPK_CASE(2)
-        MA_TOPK_CASE(5)
-        MA_TOPK_CASE(10)
-        MA_TOPK_CASE(16)
+        MA_TOPK_CASE(kClass0)
+        MA_TOPK_CASE(kClass1)
+        MA_TOPK_CASE(kClass2)
+        MA_TOPK_CASE(kClass3)
     }
 #undef MA_TOPK_CASE
     return MA_ERR_BLOCK_SIZE;
@@ -1024,55 +983,25 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
 
 template <class R, int QL>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
-    int rc = allow_big_lds(fused_step_kernel<R, 2, QL>, lds_bytes);
+    int rc = allow_big_lds(fused_step_kernel<R, kMinWaves, QL>, lds_bytes);
     if (rc) return rc;
-    fused_step_kernel<R, 2, QL><<<grid, kWG, lds_bytes, s>>>(P);
+    fused_step_kernel<R, kMinWaves, QL><<<grid, kWG, lds_bytes, s>>>(P);
     return launch_status();
 }
 
 template <template <int> class RT>
 static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // the hardware-sized block gets kernels with the quantisation group size compiled in
-    if (C == 10 && P.q_shift == 6) return launch_fused_one<RT<10>, 8>(grid, lds_bytes, s, P);
-    if (C == 10 && P.q_shift == 5) return launch_fused_one<RT<10>, 4>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 6) return launch_fused_one<RT<kClass2>, 8>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 5) return launch_fused_one<RT<kClass2>, 4>(grid, lds_bytes, s, P);
     switch (C) {
-        case 2: return launch_fused_one<RT<2>, 0>(grid, lds_bytes, s, P);
-        case 5: return launch_fused_one<RT<5>, 0>(grid, lds_bytes, s, P);
-        case 10: return launch_fused_one<RT<10>, 0>(grid, lds_bytes, s, P);
-        case 16: return launch_fused_one<RT<16>, 0>(grid, lds_bytes, s, P);
+        case kClass0: return launch_fused_one<RT<kClass0>, 0>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0>(grid, lds_bytes, s, P);
     }
     return MA_ERR_BLOCK_SIZE;
 }
-
-// Persistent launch over full blocks of the hardware block size (2048 * 10 elements): as many
-// workgroups as the device keeps resident, each walking the work items with that stride.
-template <class R, int QL>
-static int launch_persistent_one(int64_t items, int lds_bytes, hipStream_t s,
-                                 const FusedParams &P) {
-    int rc = allow_big_lds(fused_step_persistent<R, 2, QL>, lds_bytes);
-    if (rc) return rc;
-    int per_cu = 0;
-    rc = (int)hipOccupancyMaxActiveBlocksPerMultiprocessor(
-        &per_cu, reinterpret_cast<const void *>(fused_step_persistent<R, 2, QL>), kWG,
-        (size_t)lds_bytes);
-    if (rc) return rc;
-    if (per_cu < 1) per_cu = 1;
-    const int cus = ma_get_sm_count();
-    if (cus <= 0) return (int)hipErrorNoDevice;
-    int64_t grid = (int64_t)cus * per_cu;
-    if (grid > items) grid = items;
-    fused_step_persistent<R, 2, QL><<<(unsigned)grid, kWG, lds_bytes, s>>>(P);
-    return launch_status();
-}
-
-template <template <int> class RT>
-static int launch_persistent(int64_t items, int lds_bytes, hipStream_t s, const FusedParams &P) {
-    if (P.q_shift == 6) return launch_persistent_one<RT<10>, 8>(items, lds_bytes, s, P);
-    if (P.q_shift == 5) return launch_persistent_one<RT<10>, 4>(items, lds_bytes, s, P);
-    return launch_persistent_one<RT<10>, 0>(items, lds_bytes, s, P);
-}
-
-constexpr int kPersistentChunks = 10;  // the persistent kernel exists for 20480-element bf16 blocks
 
 // geometry of one tensor, micro_adam.py:77-82
 struct Geometry {
@@ -1320,15 +1249,13 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
     const int slot_bytes = h->dtype == MA_BF16 ? 2 : 4;
 
     // Work is handed out in launches of at most kTensorsPerLaunch tensors (their descriptors
-    // travel by value).  Full blocks of the hardware block size go to the persistent,
-    // pipelined kernel; every other block (tails, short tensors, other block sizes) goes to
-    // the one-workgroup-per-block kernel of its register-tile class.
+    // travel by value), one workgroup per top-k block, grouped by register-tile class so that
+    // short tensors do not run in the largest kernel.
     const int d_block_size =
         (int)(h->d_block_size > MA_MAX_D_BLOCK ? MA_MAX_D_BLOCK : h->d_block_size);
-    static const int classes[5] = {0, 2, 5, 10, 16};  // 0: the persistent pass
-    for (int ci = 0; ci < 5; ++ci) {
+    static const int classes[4] = {kClass0, kClass1, kClass2, kClass3};
+    for (int ci = 0; ci < 4; ++ci) {
         const int C = classes[ci];
-        const bool persistent = C == 0;
         FusedParams P;
         int count = 0;
         int64_t items = 0;
@@ -1342,13 +1269,9 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
             P.q_shift = q_shift;
             P.total_items = (int32_t)items;
             if (P.L.total > kLdsLimit) return MA_ERR_LDS;
-            int rc;
-            if (persistent)
-                rc = launch_persistent<RegsBF16>(items, P.L.total, s, P);
-            else
-                rc = h->dtype == MA_BF16
-                         ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
-                         : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
+            const int rc = h->dtype == MA_BF16
+                               ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
+                               : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
             count = 0;
             items = 0;
             dbs_max = kb_max = 0;
@@ -1357,19 +1280,8 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
             const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
-            const bool piped = h->dtype == MA_BF16 && g.dbs == 2048 * kPersistentChunks &&
-                               g.n_full > 0 && t.d >= g.dbs;
-            int64_t blk0, nb;
-            if (persistent) {
-                if (!piped) continue;
-                blk0 = 0;
-                nb = g.n_full;
-            } else {
-                if (chunks_for(g.dbs) != C) continue;
-                blk0 = piped ? g.n_full : 0;
-                nb = g.n_full + (g.tail > 0 ? 1 : 0) - blk0;
-                if (nb == 0) continue;
-            }
+            if (chunks_for(g.dbs) != C) continue;
+            const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
             if (count == kTensorsPerLaunch || items + nb > 0x7fffffff) {
                 const int rc = flush();
                 if (rc) return rc;
@@ -1391,7 +1303,7 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
             D.neg_lr = (float)(-t.lr);
             D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
-            D.blk0 = (int32_t)blk0;
+            D.blk0 = 0;
             items += nb;
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
