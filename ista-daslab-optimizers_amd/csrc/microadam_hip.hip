@@ -872,7 +872,11 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     extern __shared__ __align__(16) unsigned char lds[];
     const int ti = find_tensor(P, (int)blockIdx.x);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
+#ifdef MA_ANALYZE_FULL_ONLY  // development aid: a listing with the full-block path alone
+    if (true) {
+#else
     if (G.n == R::kC * kRound) {
+#endif
         FusedBlock<R, true, QL> fb(P, lds);
         fb.load_params_window(G);
         fb.load_grad_inputs(G);
@@ -880,7 +884,11 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         fb.topk_and_row(G);
         fb.quantize(G);
         fb.update(G);
+#ifdef MA_ANALYZE_FULL_ONLY
+    } else if (false) {
+#else
     } else {
+#endif
         FusedBlock<R, false, QL> fb(P, lds);
         fb.load_params_window(G);
         fb.load_grad_inputs(G);
