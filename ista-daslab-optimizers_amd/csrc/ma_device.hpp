@@ -32,7 +32,10 @@ constexpr int kShPivot = 9;     // radix select: digit of the pivot bin
 constexpr int kShNeed = 10;     //               keys still to take inside it
 constexpr int kShNEq = 11;      //               keys in the pivot bin
 constexpr int kShTies = 12;     // fast top-k: tie list length
+constexpr int kShLinks = 13;    // window pass: link cells handed out
 constexpr int kShCnts = 16;     // 8 words: candidates per wave
+constexpr int kShW1 = 32;       // 16 words: beta1^age of the window rows
+constexpr int kShW2 = 48;       // 16 words: beta2^age of the window rows
 constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
 constexpr int kMaxWindow = 64;
 

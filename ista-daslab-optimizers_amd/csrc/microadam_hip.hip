@@ -233,9 +233,10 @@ struct LdsMap {
     int slot_cells;   // multiple of 8, >= longest block
     int z_cap;        // rows of z1 / z2 / coord
     int sub_len;      // coordinates handled per window pass
+    int fast_cap;     // entries the one-pass window stage has room for, 0: none
     int total;        // bytes
 };
-constexpr int kMiscBytes = 128;  // the kSh* words at the very start
+constexpr int kMiscBytes = 256;  // the kSh* words at the very start
 constexpr int kHistBytes = 257 * kHistCopies * 4;
 
 struct WindowWeights {
@@ -401,7 +402,10 @@ struct RawChunk<RegsF32<C>> {
     }
 };
 
-constexpr int kPrefetchRows = 10;  // window rows held in registers when a block row fits one pass
+// One-pass window stage: the rows * kb entries of a block are dealt out over the workgroup,
+// entry e to thread e % kWG, and requested at the start of the block.
+constexpr int kEnt = 5;        // entries per thread at most
+constexpr int kFastRows = 16;  // window rows at most: a coordinate's rows are a 16-bit mask
 
 // Where one top-k block lives: everything a stage needs to address it, copied out of the
 // launch parameters.  Wave-uniform (lives in scalar registers).
@@ -446,8 +450,8 @@ struct FusedBlock {
     PhaseTimer pt;
 
     RawChunk<R> praw[C];          // parameters              load_params_window -> update
-    uint32_t entI[kPrefetchRows];  // older window rows, kept as loaded so that nothing waits
-    uint32_t entV[kPrefetchRows];  // for them before use     load_params_window -> update
+    uint32_t entI[kEnt];          // entries of the older window rows, kept as loaded so that
+    uint32_t entV[kEnt];          // nothing waits for them    load_params_window -> update
     RawChunk<R> graw[C];          // gradient                load_grad_inputs   -> dequant
     // 4-bit codes and statistics                            load_grad_inputs   -> dequant
     // With a full block and a compile-time quantisation group the wave's statistics are
@@ -481,7 +485,7 @@ struct FusedBlock {
     }
 
     __device__ __forceinline__ bool fast_window(const BlockGeo &G) const {
-        return G.kb <= kWG && P.W.rows <= kPrefetchRows && P.L.sub_len >= G.n;
+        return P.W.rows * G.kb <= P.L.fast_cap && P.W.rows <= kFastRows && P.L.sub_len >= G.n;
     }
 
     // ---- parameters and the older window rows: requested early, consumed last
@@ -491,18 +495,27 @@ struct FusedBlock {
 #pragma unroll
         for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
         const bool fw = fast_window(G);
-        const int rows = P.W.rows;
+        const int entries = fw ? P.W.rows * G.kb : 0;
+        const float rkb = __builtin_amdgcn_rcpf((float)G.kb);
 #pragma unroll
-        for (int row = 0; row < kPrefetchRows; ++row) {
-            entI[row] = entV[row] = 0;
-            if (fw && row < rows && row != G.D.row && tid < G.kb) {
-                const uint16_t *Ir =
-                    reinterpret_cast<const uint16_t *>(G.D.I) + ((int64_t)row * G.D.k + G.col0);
-                const uint16_t *Vr = G.D.V + ((int64_t)row * G.D.k + G.col0);
-                entI[row] = Ir[(unsigned)tid];
-                entV[row] = Vr[(unsigned)tid];
+        for (int i = 0; i < kEnt; ++i) {
+            entI[i] = entV[i] = 0;
+            if (__builtin_amdgcn_readfirstlane(wave) * kWave + i * kWG < entries) {
+                const int e = tid + i * kWG;
+                const int row = entry_row(e, rkb);
+                if (e < entries && row != G.D.row) {
+                    const int64_t at = (int64_t)row * G.D.k + G.col0 + (e - row * G.kb);
+                    entI[i] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
+                    entV[i] = G.D.V[at];
+                }
             }
         }
+    }
+
+    // row of window entry e when a row has 1 / rkb entries: (e + 0.5) / kb is at least 0.5 / kb
+    // away from an integer, far more than the rounding of the two operations
+    static __device__ __forceinline__ int entry_row(int e, float rkb) {
+        return (int)(((float)e + 0.5f) * rkb);
     }
 
     // ---- gradient, 4-bit error feedback and its statistics
@@ -730,55 +743,112 @@ struct FusedBlock {
 #else
         if (fast_window(G)) {
 #endif
-            // One entry per thread and row.  Entry (row, tid) owns row*kb + tid of z1 / z2 /
-            // coord; the first entry (in row order) to name a coordinate becomes its owner
-            // and later rows add into the owner's sums.  Rows are separated by barriers and a
-            // row never names a coordinate twice, so the sums are formed in row order.
+            // Every entry of the window is handled once, kEnt per thread.  The rows that name
+            // a coordinate are first gathered as a bit mask in its slot cell.  A coordinate
+            // named by one row gets its update from that entry alone.  The entries of the
+            // others go to a list; the entry of the lowest row owns the coordinate, hands out
+            // one link cell per later row, the later rows file their list position there by
+            // rank, and the owner adds them up in that order, which is the order of the rows.
+            uint32_t *mcount = sh + kShCounter, *lcount = sh + kShLinks;
+            float *f1 = z1, *f2 = z2;
+            const int cap = P.L.z_cap;
+            uint16_t *mI = coord, *mR = mI + cap, *mM = mR + cap, *link = mM + cap;
+            if (tid < kFastRows) {
+                sh[kShW1 + tid] = __float_as_uint(P.W.w1[tid]);
+                sh[kShW2 + tid] = __float_as_uint(P.W.w2[tid]);
+            }
+            if (tid == 0) *mcount = *lcount = 0;
+            const int wave_first = __builtin_amdgcn_readfirstlane(wave) * kWave;
+            const int entries = rows * kb;
+            const float rkb = __builtin_amdgcn_rcpf((float)kb);
             __syncthreads();
             pt.mark(12);
 #pragma unroll
-            for (int row = 0; row < kPrefetchRows; ++row) {
-                if (row < rows) {
-                    int idx = (int)entI[row];
-                    uint32_t vb = entV[row];
-                    if (row == D.row && tid < kb) {
-                        idx = sel_idx[tid];
-                        vb = sel_val[tid];
-                    }
-                    // +-0 values add nothing and are skipped (the rows of a fresh window are
-                    // all (index 0, value 0)); idx < n also keeps a corrupt index inside
-                    const bool active = tid < kb && idx < n && (vb & 0x7fffu) != 0;
-                    const int own = row * kb + tid;
-                    if (tid < kb) {
-                        const float v = bf2f(vb);
-                        const float a1 = P.W.w1[row] * v;
-                        const float vv = v * v;
-                        const float a2 = P.W.w2[row] * vv;
-                        uint32_t owner_idx = 0xffffu;
-                        if (active) {
-                            const uint32_t s = slot[idx];
-                            if (s == 0) {
-                                slot[idx] = (slot_t)(own + 1);
-                                z1[own] = 0.0f + a1;
-                                z2[own] = 0.0f + a2;
-                                owner_idx = (uint32_t)idx;
-                            } else {
-                                z1[s - 1] = z1[s - 1] + a1;
-                                z2[s - 1] = z2[s - 1] + a2;
-                            }
+            for (int i = 0; i < kEnt; ++i) {
+                uint32_t tag = 0xffffffffu;  // index | row << 16, all ones: nothing to add
+                if (wave_first + i * kWG < entries) {
+                    const int e = tid + i * kWG;
+                    const int row = entry_row(e, rkb);
+                    if (e < entries) {
+                        uint32_t idx = entI[i], vb = entV[i];
+                        if (row == D.row) {
+                            idx = sel_idx[e - row * kb];
+                            vb = sel_val[e - row * kb];
+                            entV[i] = vb;
                         }
-                        coord[own] = (uint16_t)owner_idx;
+                        // +-0 values add nothing and are skipped (the rows of a fresh window
+                        // are all (index 0, value 0)); idx < n keeps a corrupt index inside
+                        if (idx < (uint32_t)n && (vb & 0x7fffu) != 0) {
+                            tag = idx | (uint32_t)row << 16;
+                            if (sizeof(slot_t) == 2)
+                                atomicOr(reinterpret_cast<uint32_t *>(slot) + (idx >> 1),
+                                         (1u << row) << ((idx & 1u) * 16));
+                            else
+                                atomicOr(reinterpret_cast<uint32_t *>(slot) + idx, 1u << row);
+                        }
                     }
-                    __syncthreads();
+                }
+                entI[i] = tag;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kEnt; ++i) {
+                const uint32_t tag = entI[i];
+                if (tag != 0xffffffffu) {
+                    const uint32_t idx = tag & 0xffffu, row = tag >> 16;
+                    const uint32_t mask = slot[idx];
+                    const float v = bf2f(entV[i]);
+                    const float a1 = __uint_as_float(sh[kShW1 + row]) * v;
+                    const float vv = v * v;
+                    const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
+                    if (mask == 1u << row) {
+                        const float u =
+                            adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                        slot[idx] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                    } else {
+                        const uint32_t s = atomicAdd(mcount, 1u);
+                        f1[s] = a1;
+                        f2[s] = a2;
+                        mI[s] = (uint16_t)idx;
+                        mR[s] = (uint16_t)row;
+                        mM[s] = (uint16_t)mask;
+                    }
                 }
             }
+            __syncthreads();
             pt.mark(13);
-            const int entries = rows * kb;
-            for (int s = tid; s < entries; s += kWG) {
-                const uint32_t ci = coord[s];
-                if (ci != 0xffffu) {
-                    const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
-                    slot[ci] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+            const int listed = (int)(*mcount < (uint32_t)cap ? *mcount : (uint32_t)cap);
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below == 0)
+                    slot[mI[s]] = (slot_t)atomicAdd(lcount, (uint32_t)__popc(mask) - 1u);
+            }
+            __syncthreads();
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below != 0) {
+                    const uint32_t at = (uint32_t)slot[mI[s]] + (uint32_t)__popc(below) - 1u;
+                    if (at < (uint32_t)cap) link[at] = (uint16_t)s;
+                }
+            }
+            __syncthreads();
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below == 0) {
+                    const uint32_t idx = mI[s], base = slot[idx];
+                    float s1 = 0.0f + f1[s], s2 = 0.0f + f2[s];
+                    const int later = __popc(mask) - 1;
+                    for (int r = 0; r < later; ++r) {
+                        // a valid window keeps base + r and the link inside the list
+                        uint32_t at = base + (uint32_t)r;
+                        at = at < (uint32_t)cap ? at : (uint32_t)cap - 1u;
+                        uint32_t o = link[at];
+                        o = o < (uint32_t)cap ? o : (uint32_t)cap - 1u;
+                        s1 = s1 + f1[o];
+                        s2 = s2 + f2[o];
+                    }
+                    const float u = adam_direction(s1, s2, P.W.s1, P.W.s2, P.W.eps);
+                    slot[idx] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
                 }
             }
             __syncthreads();
@@ -922,7 +992,10 @@ static LdsMap plan_lds(int dbs_max, int kb_max, int m, int slot_bytes) {
         L.sub_len = 4096;
         L.z_cap = 4096;
     }
-    const int zbytes = L.z_cap * 10;
+    // one-pass window stage: two floats and four 16-bit words per entry
+    L.fast_cap = 0;
+    if (entries <= kEnt * kWG && m <= kFastRows) L.fast_cap = L.z_cap;
+    const int zbytes = L.z_cap * (L.fast_cap ? 16 : 10);
     L.total = L.off_union + align16(zbytes > kHistBytes ? zbytes : kHistBytes);
     return L;
 }
