@@ -34,6 +34,8 @@ constexpr int kShNEq = 11;      //               keys in the pivot bin
 constexpr int kShTies = 12;     // fast top-k: tie list length
 constexpr int kShLinks = 13;    // window pass: link cells handed out
 constexpr int kShCnts = 16;     // 8 words: candidates per wave
+constexpr int kShSel = 24;      // 8 words: (pivot digit, keys still to take) per radix pass of
+                                //          the two selections of the fast top-k
 constexpr int kShW1 = 32;       // 16 words: beta1^age of the window rows
 constexpr int kShW2 = 48;       // 16 words: beta2^age of the window rows
 constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
@@ -408,17 +410,16 @@ constexpr int kSmallHistWords = 2 * 257 * kSmallCopies;  // one histogram per pa
 // histogram; wave 0 alone then walks the 256 bins from the top (4 bins per lane, a DPP prefix
 // sum across lanes) and publishes the digit that holds the kb-th key, which costs two
 // barriers per pass instead of a workgroup-wide scan.
-//   hist: kSmallHistWords words, sh: 8 words.  Ends with a barrier.
+//   hist: kSmallHistWords words, all zero, and all threads past the barrier that says so;
+//   shp: 4 words of its own per call.  Ends with the barrier after the second walk: a caller
+//   that uses the same hist / shp words again puts a barrier in between.
 //   valid: bit i set if v[i] takes part.  take_eq: how many keys equal to the result belong
 //   to the top kb; n_eq: how many keys equal it in all.
 template <int N>
 __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uint32_t valid,
-                                                     int kb, uint32_t *hist, uint32_t *sh,
-                                                     int &take_eq, int &n_eq) {
+                                                     int kb, uint32_t *hist, uint32_t *shp,
+                                                     uint32_t *sh_neq, int &take_eq, int &n_eq) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < kSmallHistWords / 4; i += kWG)
-        reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
-    __syncthreads();
     uint32_t prefix = 0, pmask = 0;
     int need = kb;
 #pragma unroll
@@ -450,22 +451,21 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (above < (uint32_t)need && (uint32_t)need <= above + c[i]) {
-                        sh[kShPivot] = (uint32_t)(255 - 4 * lane - i);
-                        sh[kShNeed] = (uint32_t)need - above;
-                        sh[kShNEq] = c[i];
+                        shp[2 * pass] = (uint32_t)(255 - 4 * lane - i);
+                        shp[2 * pass + 1] = (uint32_t)need - above;
+                        *sh_neq = c[i];
                     }
                     above += c[i];
                 }
             }
         }
         __syncthreads();
-        prefix |= sh[kShPivot] << shift;
+        prefix |= shp[2 * pass] << shift;
         pmask |= dm << shift;
-        need = (int)sh[kShNeed];
+        need = (int)shp[2 * pass + 1];
     }
     take_eq = need;
-    n_eq = (int)sh[kShNEq];
-    __syncthreads();
+    n_eq = (int)*sh_neq;
     return prefix;
 }
 
@@ -475,7 +475,8 @@ constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multi
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
 // magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false
 // (a wave found more candidates than it has room for: heavy ties) r is reloaded unchanged.
-//   hist: kSmallHistWords + 4*kCandPerWave words; sh: 16 words.  1 <= kb <= 256.
+//   hist: 2*kSmallHistWords + kWaves*kCandPerWave words; sh: the kSh* words.  1 <= kb <= 256.
+//   On success every thread has also cleared the cells of `park` that hold its own chunks.
 // Output order: entries above the threshold key in candidate-list order, then the kept
 // entries equal to it by increasing index; deterministic for given data.
 template <class R>
@@ -484,7 +485,11 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
                                                uint16_t *sel_val, PhaseTimer &pt) {
     constexpr int C = R::kC;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
-    uint32_t *cand = hist + kSmallHistWords;
+    uint32_t *cand = hist + 2 * kSmallHistWords;
+    // the histograms of both selections are cleared here, under the one barrier that also
+    // covers the parked block
+    for (int i = tid; i < 2 * kSmallHistWords / 4; i += kWG)
+        reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
     uint32_t cmax[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) {
@@ -493,9 +498,11 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
             make_uint4(r.w[c][0], r.w[c][1], r.w[c][2], r.w[c][3]);
         cmax[c] = chunk_max_key(r.w[c]);
     }
+    __syncthreads();
     pt.mark(1);
     int unused_take, unused_eq;
-    const uint32_t L = select_kth_key15<C>(cmax, 0xffffffffu, kb, hist, sh, unused_take, unused_eq);
+    const uint32_t L = select_kth_key15<C>(cmax, 0xffffffffu, kb, hist, sh + kShSel,
+                                           sh + kShNEq, unused_take, unused_eq);
     pt.mark(2);
 
     // candidates: every element with key >= L, wave by wave into the wave's own list
@@ -569,8 +576,9 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         const uint32_t keys[2] = {my[0] >> 15, my[1] >> 15};
         if (tid == 0) sh[kShTies] = 0;
         int take_eq, n_eq;
-        const uint32_t T = select_kth_key15<2>(keys, have, kb, hist, sh, take_eq, n_eq);
-        uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the histogram is free again
+        const uint32_t T = select_kth_key15<2>(keys, have, kb, hist + kSmallHistWords,
+                                               sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
+        uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the first histograms are free
         constexpr int kMaxTies = 512;
         ok = n_eq <= kMaxTies;
         if (ok) {
@@ -620,6 +628,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         r.w[c][1] = q.y;
         r.w[c][2] = q.z;
         r.w[c][3] = q.w;
+        if (ok) *reinterpret_cast<uint4 *>(park + off) = make_uint4(0, 0, 0, 0);
     }
     return ok;
 }

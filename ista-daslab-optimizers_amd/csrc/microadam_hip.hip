@@ -237,7 +237,9 @@ struct LdsMap {
     int total;        // bytes
 };
 constexpr int kMiscBytes = 256;  // the kSh* words at the very start
-constexpr int kHistBytes = 257 * kHistCopies * 4;
+constexpr int kFastTopkBytes = (2 * kSmallHistWords + 512) * 4;
+constexpr int kHistBytes =
+    257 * kHistCopies * 4 > kFastTopkBytes ? 257 * kHistCopies * 4 : kFastTopkBytes;
 
 struct WindowWeights {
     float w1[kMaxWindow];
@@ -446,6 +448,7 @@ struct FusedBlock {
     slot_t *slot;
     float *z1, *z2;
     int tid, lane, wave, q_shift, ql;
+    bool slot_clear;  // the slot cells are already zero when the update stage begins
     Divisor d15;
     PhaseTimer pt;
 
@@ -481,6 +484,7 @@ struct FusedBlock {
         // 1/15 rounded to nearest; div_shared is exact for a reciprocal within one ulp
         d15.u = 15.0f;
         d15.r = 0x1.111112p-4f;
+        slot_clear = false;
         pt.begin();
     }
 
@@ -617,6 +621,8 @@ struct FusedBlock {
                                            sel_idx, sel_val, pt);
                 launder(r);
                 pt.mark(7);
+                // the block was parked in the slot cells and every thread cleared its own
+                slot_clear = topk_done && P.L.slot_cells == C * kRound;
             }
         }
         if (!topk_done) {
@@ -735,9 +741,11 @@ struct FusedBlock {
         const int kb = G.kb;
         const int rows = P.W.rows;
         const TensorDesc &D = G.D;
-        __syncthreads();  // the LDS of the selection is reused below
-        for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
-            reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+        if (!slot_clear) {
+            __syncthreads();  // the LDS of the selection is reused below
+            for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
+                reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+        }
 #if defined(MA_ABLATE) && MA_ABLATE == 3
         if (false) {
 #else
