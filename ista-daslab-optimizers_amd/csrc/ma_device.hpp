@@ -1,7 +1,7 @@
 // Device-side building blocks of the MicroAdam step for gfx950 (wave64, 160 KB LDS per CU).
 //
-// One workgroup of 256 threads (4 waves, one per SIMD) owns one top-k block of up to
-// 2048*C elements and keeps it in VGPRs for the whole step.  Wave w, chunk c, lane l holds
+// One workgroup of kWG = 512 threads (8 waves, two per SIMD) owns one top-k block of up to
+// kRound*C = 4096*C elements and keeps it in VGPRs for the whole step.  Wave w, chunk c, lane l holds
 // the 8 consecutive elements starting at ((w*C + c)*64 + l)*8, so every 128-bit load of a
 // wave covers one contiguous KiB (bf16) and the block's index order is (wave, chunk, lane,
 // element).  Elements past the block's length read as +0.0, which the lowest-index tie rule
@@ -65,9 +65,9 @@ struct PhaseTimer {
 };
 #endif
 
-// The thread id as a value the optimiser cannot see through.  Stages that run inside a
-// persistent loop derive their lane offsets from this, so that the offsets are rebuilt where
-// they are used instead of being hoisted out of the loop into long-lived registers.
+// The thread id as a value the optimiser cannot see through.  The selection helpers derive
+// their lane offsets from this, so that the offsets are rebuilt where they are used instead
+// of being computed once and kept in long-lived registers.
 __device__ __forceinline__ int opaque_tid() {
     int t = (int)threadIdx.x;
     asm volatile("" : "+v"(t));
@@ -161,7 +161,7 @@ __device__ __forceinline__ void group_minmax(float &mn, float &mx, int ql_runtim
     }
 }
 
-// Inclusive scan over the 256 threads in thread order.  sh4 is 4 words of LDS.
+// Inclusive scan over the workgroup in thread order.  sh4 is kWaves words of LDS.
 __device__ __forceinline__ uint32_t wg_incl_scan(uint32_t v, uint32_t *sh4, int lane, int wave) {
     uint32_t s = wave_incl_scan(v, lane);
     if (lane == kWave - 1) sh4[wave] = s;
@@ -182,7 +182,7 @@ struct RegsBF16 {
     static constexpr bool kBF16 = true;
     static constexpr int kElemBytes = 2;
     typedef uint16_t elem_t;
-    typedef uint16_t slot_t;  // LDS cell that first holds a slot id, later the update's bits
+    typedef uint16_t slot_t;  // LDS cell per coordinate: window bookkeeping, later the update's bits
     uint32_t w[C][4];         // two bf16 per register
 
     __device__ __forceinline__ uint32_t key(int c, int e) const {
@@ -471,7 +471,7 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 
 constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multiple of 16); more falls back
 
-// The fast top-k of a full bf16 block.  `park` (2048*C uint16 cells) receives the block;
+// The fast top-k of a full bf16 block.  `park` (kRound*C uint16 cells) receives the block;
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
 // magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false
 // (a wave found more candidates than it has room for: heavy ties) r is reloaded unchanged.

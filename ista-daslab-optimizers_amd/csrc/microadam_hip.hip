@@ -229,9 +229,9 @@ struct LdsMap {
     int off_sel_idx;  // uint16[kb_max]
     int off_sel_val;  // uint16[kb_max]
     int off_slot;     // slot_t[slot_cells]
-    int off_union;    // histogram (32 KiB) during selection, then z1 | z2 | coord
+    int off_union;    // histograms and candidate lists during selection, then the window stage's arrays
     int slot_cells;   // multiple of 8, >= longest block
-    int z_cap;        // rows of z1 / z2 / coord
+    int z_cap;        // entries the window stage's arrays hold
     int sub_len;      // coordinates handled per window pass
     int fast_cap;     // entries the one-pass window stage has room for, 0: none
     int total;        // bytes
@@ -434,7 +434,7 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
 
 // The step of one block, cut into stages.  The register arrays are members; the stages say
 // which of them they fill and which they consume.
-//   FULL: the block has exactly 2048*C elements, so no chunk needs a bounds check.
+//   FULL: the block has exactly kRound*C elements, so no chunk needs a bounds check.
 //   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
 template <class R, bool FULL, int QL>
 struct FusedBlock {
