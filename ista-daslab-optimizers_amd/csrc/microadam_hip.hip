@@ -347,6 +347,7 @@ struct TensorDesc {
     float decay;
     int32_t apply_decay;
     int32_t blk0;         // block of the tensor that its first work item stands for
+    uint16_t *ws;         // three-pass route: per-block partial statistics, else unused
 };
 constexpr int kTensorsPerLaunch = 24;
 
@@ -358,6 +359,10 @@ struct FusedParams {
     int32_t d_block_size;
     int32_t q_shift;  // log2(quant_block_size)
     int32_t total_items;  // work items (blocks) of the launch
+    // three-pass route (quantisation blocks at least as long as the top-k blocks)
+    int32_t q_span;   // quantisation block length, a multiple of 8
+    float alpha;      // share of the dequantised error feedback added to the update
+    float keep;       // (float)(1 - alpha): share that stays in the error feedback
 };
 
 template <class R>
@@ -449,6 +454,7 @@ struct FusedBlock {
     float *z1, *z2;
     int tid, lane, wave, q_shift, ql;
     bool slot_clear;  // the slot cells are already zero when the update stage begins
+    bool row_in_lds;  // the window row of this step is taken from sel_idx / sel_val, not from HBM
     Divisor d15;
     PhaseTimer pt;
 
@@ -485,6 +491,7 @@ struct FusedBlock {
         d15.u = 15.0f;
         d15.r = 0x1.111112p-4f;
         slot_clear = false;
+        row_in_lds = true;
         pt.begin();
     }
 
@@ -507,7 +514,7 @@ struct FusedBlock {
             if (__builtin_amdgcn_readfirstlane(wave) * kWave + i * kWG < entries) {
                 const int e = tid + i * kWG;
                 const int row = entry_row(e, rkb);
-                if (e < entries && row != G.D.row) {
+                if (e < entries && (row != G.D.row || !row_in_lds)) {
                     const int64_t at = (int64_t)row * G.D.k + G.col0 + (e - row * G.kb);
                     entI[i] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
                     entV[i] = G.D.V[at];
@@ -737,6 +744,13 @@ struct FusedBlock {
     //      and p += -lr * u (MA:304).  The slot cells end up holding the update's bits, 0
     //      where no window row names the coordinate.
     __device__ __forceinline__ void update(const BlockGeo &G) {
+        window_stage(G);
+        param_stage(G);
+    }
+
+    // The slot cells end up holding the update's bits, 0 where no window row names the
+    // coordinate.  Ends with a barrier.
+    __device__ __forceinline__ void window_stage(const BlockGeo &G) {
         const int n = FULL ? C * kRound : G.n;
         const int kb = G.kb;
         const int rows = P.W.rows;
@@ -779,7 +793,7 @@ struct FusedBlock {
                     const int row = entry_row(e, rkb);
                     if (e < entries) {
                         uint32_t idx = entI[i], vb = entV[i];
-                        if (row == D.row) {
+                        if (row == D.row && row_in_lds) {
                             idx = sel_idx[e - row * kb];
                             vb = sel_val[e - row * kb];
                             entV[i] = vb;
@@ -871,7 +885,7 @@ struct FusedBlock {
             wv.V = D.V + G.col0;
             wv.k = D.k;
             wv.rows = rows;
-            wv.cur_row = D.row;
+            wv.cur_row = row_in_lds ? D.row : -1;
             wv.cur_idx = sel_idx;
             wv.cur_val = sel_val;
             wv.w1 = P.W.w1;
@@ -889,7 +903,11 @@ struct FusedBlock {
             }
         }
         pt.mark(15);
+    }
 
+    __device__ __forceinline__ void param_stage(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
         const bool apply_decay = D.apply_decay != 0;
@@ -933,6 +951,373 @@ struct FusedBlock {
         }
         pt.mark(16);
     }
+
+    // =========================================================================================
+    // Three-pass route: quantisation blocks of q_span >= block length elements (q_span a
+    // multiple of 8), so a top-k block meets at most two of them and their statistics need
+    // every top-k block they cover.  alpha > 0 (MA:296-298, 311-316).
+    //   pass 1: a = g + Qinv(e), top-k, window row; the residual r goes to the gradient
+    //           buffer, its min / max per (block, segment) to the workspace (set 0)
+    //   pass 2: e1 = Q(r), d1 = Qinv(e1) in registers; u = Adam(window) + alpha * d1;
+    //           p update; min / max of r2 = (1 - alpha) * d1 to the workspace (set 1)
+    //   pass 3: r2 again from r, e = Q(r2), statistics arrays
+    // Segment 0 of a block is its part in the quantisation block of its first element,
+    // segment 1 the rest.  Workspace: 4 bf16 words (min0, max0, min1, max1) per block and set.
+    // =========================================================================================
+    struct Span {
+        int64_t qb0;  // quantisation block of the block's first element
+        int bnd;      // offset inside the block where the next one starts, INT_MAX if it does not
+    };
+
+    __device__ __forceinline__ Span make_span(const BlockGeo &G) const {
+        const int n = FULL ? C * kRound : G.n;
+        Span S;
+        const int64_t q = P.q_span;
+        S.qb0 = G.e0 / q;
+        const int64_t rel = (S.qb0 + 1) * q - G.e0;
+        S.bnd = rel < n ? (int)rel : 0x7fffffff;
+        return S;
+    }
+
+    __device__ __forceinline__ int64_t block_id(const BlockGeo &G) const {
+        const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
+        return G.e0 / dbs;
+    }
+
+    // min / max over the workgroup of two pairs; every thread gets the result.  Uses the 32
+    // words at kShW1 and two barriers.
+    __device__ __forceinline__ void wg_minmax2(float (&mn)[2], float (&mx)[2]) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) group_minmax<0>(mn[s2], mx[s2], kWave);
+        __syncthreads();
+        if (lane == 0) {
+            sh[kShW1 + wave * 4 + 0] = __float_as_uint(mn[0]);
+            sh[kShW1 + wave * 4 + 1] = __float_as_uint(mx[0]);
+            sh[kShW1 + wave * 4 + 2] = __float_as_uint(mn[1]);
+            sh[kShW1 + wave * 4 + 3] = __float_as_uint(mx[1]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mn[0] = fmin_raw(mn[0], __uint_as_float(sh[kShW1 + w * 4 + 0]));
+            mx[0] = fmax_raw(mx[0], __uint_as_float(sh[kShW1 + w * 4 + 1]));
+            mn[1] = fmin_raw(mn[1], __uint_as_float(sh[kShW1 + w * 4 + 2]));
+            mx[1] = fmax_raw(mx[1], __uint_as_float(sh[kShW1 + w * 4 + 3]));
+        }
+    }
+
+    __device__ __forceinline__ void store_partials(const BlockGeo &G, int set, float (&mn)[2],
+                                                   float (&mx)[2]) {
+        wg_minmax2(mn, mx);
+        if (tid == 0) {
+            uint16_t *w = G.D.ws + (block_id(G) * 2 + set) * 4;
+            w[0] = (uint16_t)f2bf(mn[0]);
+            w[1] = (uint16_t)f2bf(mx[0]);
+            w[2] = (uint16_t)f2bf(mn[1]);
+            w[3] = (uint16_t)f2bf(mx[1]);
+        }
+    }
+
+    // statistics (bf16 bits) of the two quantisation blocks this top-k block meets, from the
+    // partials of all top-k blocks that cover them (at most 64 each: lane i takes one)
+    __device__ __forceinline__ void gather_stats(const BlockGeo &G, const Span &S, int set,
+                                                 uint32_t (&mnb)[2], uint32_t (&mxb)[2]) const {
+        const int64_t q = P.q_span;
+        const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
+        const int64_t nblk = (G.D.d + dbs - 1) / dbs;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            float mn = INFINITY, mx = -INFINITY;
+            if (s2 == 0 || S.bnd != 0x7fffffff) {
+                const int64_t Q = S.qb0 + s2;
+                const int64_t first = Q * q;
+                const int64_t b_lo = first / dbs;
+                int64_t b_hi = (first + q - 1) / dbs;
+                b_hi = b_hi < nblk - 1 ? b_hi : nblk - 1;
+                const int64_t b = b_lo + lane;
+                if (b <= b_hi) {
+                    const int seg = b * dbs >= first ? 0 : 1;
+                    const uint16_t *w = G.D.ws + (b * 2 + set) * 4 + seg * 2;
+                    mn = bf2f(w[0]);
+                    mx = bf2f(w[1]);
+                }
+                group_minmax<0>(mn, mx, kWave);
+            }
+            mnb[s2] = f2bf(mn);
+            mxb[s2] = f2bf(mx);
+        }
+    }
+
+    // 4-bit codes of 8 values against (mn, u) as small exact floats: floor((x - mn)/u + 0.5)
+    // clamped to [0, 15]; all zero when the range is zero or not finite.  Same arithmetic as
+    // the quantize stage.
+    __device__ __forceinline__ void codes8(const float (&x)[8], float mnf, float u,
+                                           float (&cf)[8]) const {
+        const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
+        const float lim = 32.0f * u;
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            y[e] = x[e] - mnf;
+            if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
+        }
+        bool ok = true;
+        float us = u;
+        if (ex - 32u > 190u) {
+            ok = u != 0.0f && isfinite(u);
+            const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
+            us = ok ? u * sc : 1.0f;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
+        }
+        const Divisor dv = make_divisor(us);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            float v = div_shared(y[e], dv);
+            v = floorf(v + 0.5f);
+            v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+            cf[e] = ok ? v : 0.0f;
+        }
+    }
+
+    // two 16-bit halves, nibble order (e0 e1)(e2 e3) | (e4 e5)(e6 e7), even element high
+    static __device__ __forceinline__ uint32_t pack_codes(const float (&cf)[8]) {
+        float lo = cf[2];
+        lo = __builtin_fmaf(lo, 16.0f, cf[3]);
+        lo = __builtin_fmaf(lo, 16.0f, cf[0]);
+        lo = __builtin_fmaf(lo, 16.0f, cf[1]);
+        float hi = cf[6];
+        hi = __builtin_fmaf(hi, 16.0f, cf[7]);
+        hi = __builtin_fmaf(hi, 16.0f, cf[4]);
+        hi = __builtin_fmaf(hi, 16.0f, cf[5]);
+        return (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+
+    static __device__ __forceinline__ float to_elem(float v) {
+        return R::kBF16 ? bf2f(f2bf(v)) : v;
+    }
+
+    // ---- pass 1 ------------------------------------------------------------------------------
+    uint32_t sp_mn[2], sp_mx[2];  // statistics of the two segments (bf16 bits), wave-uniform
+
+    __device__ __forceinline__ void span_load_grad_inputs(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+        const uint8_t *err = G.D.err + (G.e0 >> 1);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            graw[c].load(g, off, n, FULL);
+            cw[c] = 0;
+            if (FULL || off < n) {
+                if (FULL || off + kChunk <= n) {
+                    cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        cw[c] |= (uint32_t)err[(off >> 1) + j] << (8 * j);
+                }
+            }
+        }
+        sp_mn[0] = G.D.mn[S.qb0];
+        sp_mx[0] = G.D.mx[S.qb0];
+        sp_mn[1] = sp_mx[1] = 0;
+        if (S.bnd != 0x7fffffff) {
+            sp_mn[1] = G.D.mn[S.qb0 + 1];
+            sp_mx[1] = G.D.mx[S.qb0 + 1];
+        }
+    }
+
+    __device__ __forceinline__ void span_dequant(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float v[8];
+            graw[c].to_float(v);
+            const bool second = off >= S.bnd;
+            const float mn = second ? mn1 : mn0, u = second ? u1 : u0;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                float deq = (float)code * u;
+                deq = deq + mn;
+                v[e] = v[e] + deq;
+            }
+            if (!FULL && off + kChunk > n) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (off + e >= n) v[e] = 0.0f;
+            }
+            r.set_chunk(c, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        launder(r);
+    }
+
+    // the residual goes to the gradient buffer (which the step may destroy, MA:190-214 does)
+    __device__ __forceinline__ void span_store_residual(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        elem_t *out = reinterpret_cast<elem_t *>(const_cast<void *>(G.D.g)) + G.e0;
+        float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float x[8];
+                float lmn = INFINITY, lmx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    x[e] = r.val(c, e);
+                    if (FULL || off + e < n) {
+                        lmn = fmin_raw(lmn, x[e]);
+                        lmx = fmax_raw(lmx, x[e]);
+                    }
+                }
+                const bool second = off >= S.bnd;
+                mn[0] = fmin_raw(mn[0], second ? INFINITY : lmn);
+                mx[0] = fmax_raw(mx[0], second ? -INFINITY : lmx);
+                mn[1] = fmin_raw(mn[1], second ? lmn : INFINITY);
+                mx[1] = fmax_raw(mx[1], second ? lmx : -INFINITY);
+                store8(out, off, FULL ? 0x7fffffff : n, true, x);
+            }
+        }
+        store_partials(G, 0, mn, mx);
+    }
+
+    // ---- pass 2 and 3 -----------------------------------------------------------------------
+    __device__ __forceinline__ void span_load_residual(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) graw[c].load(g, chunk_off<C>(wave, c, lane), n, FULL);
+    }
+
+    // d1 = Qinv(Q(r)) of one chunk, (float)code * u + mn as in span_dequant
+    __device__ __forceinline__ void span_requant(int c, float mnf, float u, float (&d1)[8]) {
+        float x[8], cf[8];
+        graw[c].to_float(x);
+        codes8(x, mnf, u, cf);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            float deq = cf[e] * u;
+            d1[e] = deq + mnf;
+        }
+    }
+
+    // p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u; partial statistics of
+    // r2 = rne(0 + keep * d1).  After window_stage.
+    __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+        float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                const bool second = off >= S.bnd;
+                float d1[8];
+                span_requant(c, second ? mn1 : mn0, second ? u1 : u0, d1);
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                if (R::kBF16) {
+                    const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
+                    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        uv[2 * i] = __uint_as_float(w[i] << 16);
+                        uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                    }
+                } else {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
+                    const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
+                    uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
+                    uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
+                    uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
+                    uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
+                }
+                float lmn = INFINITY, lmx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                    const float add = P.alpha * d1[e];
+                    const float ud = to_elem(uv[e] + add);
+                    const float prod = neg_lr * ud;
+                    pv[e] = pv[e] + prod;
+                    const float keep = P.keep * d1[e];
+                    const float r2 = to_elem(0.0f + keep);
+                    if (FULL || off + e < n) {
+                        lmn = fmin_raw(lmn, r2);
+                        lmx = fmax_raw(lmx, r2);
+                    }
+                }
+                mn[0] = fmin_raw(mn[0], second ? INFINITY : lmn);
+                mx[0] = fmax_raw(mx[0], second ? -INFINITY : lmx);
+                mn[1] = fmin_raw(mn[1], second ? lmn : INFINITY);
+                mx[1] = fmax_raw(mx[1], second ? lmx : -INFINITY);
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_partials(G, 1, mn, mx);
+    }
+
+    // e = Q(r2) against the statistics of r2, and the statistics arrays themselves
+    __device__ __forceinline__ void span_final_codes(const BlockGeo &G, const Span &S,
+                                                     const uint32_t (&mn2b)[2],
+                                                     const uint32_t (&mx2b)[2]) {
+        const int n = FULL ? C * kRound : G.n;
+        uint8_t *err = G.D.err + (G.e0 >> 1);
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+        const float m20 = bf2f(mn2b[0]), m21 = bf2f(mn2b[1]);
+        const float v0 = div15(bf2f(mx2b[0]) - m20, d15), v1 = div15(bf2f(mx2b[1]) - m21, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                const bool second = off >= S.bnd;
+                float d1[8], r2[8], cf[8];
+                span_requant(c, second ? mn1 : mn0, second ? u1 : u0, d1);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    const float keep = P.keep * d1[e];
+                    r2[e] = to_elem(0.0f + keep);
+                }
+                codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the block that holds the first element of a quantisation block writes its statistics
+        if (tid == 0) {
+            if (G.e0 == S.qb0 * (int64_t)P.q_span) {
+                G.D.mn[S.qb0] = (uint16_t)mn2b[0];
+                G.D.mx[S.qb0] = (uint16_t)mx2b[0];
+            }
+            if (S.bnd != 0x7fffffff) {
+                G.D.mn[S.qb0 + 1] = (uint16_t)mn2b[1];
+                G.D.mx[S.qb0 + 1] = (uint16_t)mx2b[1];
+            }
+        }
+    }
 };
 
 // which tensor owns workgroup / work item `w` of the launch (first_block is ascending)
@@ -974,6 +1359,43 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         fb.topk_and_row(G);
         fb.quantize(G);
         fb.update(G);
+    }
+}
+
+// Three-pass route, see FusedBlock.  PASS 1 / 2 / 3; one workgroup per block.
+template <class R, int MIN_WAVES, int PASS>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int ti = find_tensor(P, (int)blockIdx.x);
+    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
+    auto run = [&](auto &fb) {
+        const auto S = fb.make_span(G);
+        if constexpr (PASS == 1) {
+            fb.span_load_grad_inputs(G, S);
+            fb.span_dequant(G, S);
+            fb.topk_and_row(G);
+            fb.span_store_residual(G, S);
+        } else if constexpr (PASS == 2) {
+            fb.row_in_lds = false;
+            fb.load_params_window(G);
+            fb.span_load_residual(G);
+            fb.gather_stats(G, S, 0, fb.sp_mn, fb.sp_mx);
+            fb.window_stage(G);
+            fb.span_param_stage(G, S);
+        } else {
+            fb.span_load_residual(G);
+            fb.gather_stats(G, S, 0, fb.sp_mn, fb.sp_mx);
+            uint32_t mn2[2], mx2[2];
+            fb.gather_stats(G, S, 1, mn2, mx2);
+            fb.span_final_codes(G, S, mn2, mx2);
+        }
+    };
+    if (G.n == R::kC * kRound) {
+        FusedBlock<R, true, 0> fb(P, lds);
+        run(fb);
+    } else {
+        FusedBlock<R, false, 0> fb(P, lds);
+        run(fb);
     }
 }
 
@@ -1092,6 +1514,40 @@ static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, cons
     return MA_ERR_BLOCK_SIZE;
 }
 
+template <class R>
+static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                           const FusedParams &P) {
+    int rc;
+    switch (pass) {
+        case 1:
+            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        case 2:
+            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        default:
+            span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
+            break;
+    }
+    return launch_status();
+}
+
+template <template <int> class RT>
+static int launch_span(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                       const FusedParams &P) {
+    switch (C) {
+        case kClass0: return launch_span_one<RT<kClass0>>(pass, grid, lds_bytes, s, P);
+        case kClass1: return launch_span_one<RT<kClass1>>(pass, grid, lds_bytes, s, P);
+        case kClass2: return launch_span_one<RT<kClass2>>(pass, grid, lds_bytes, s, P);
+        case kClass3: return launch_span_one<RT<kClass3>>(pass, grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
+}
+
 // geometry of one tensor, micro_adam.py:77-82
 struct Geometry {
     int64_t dbs, n_full, tail, k_many, k_few, k;
@@ -1107,7 +1563,8 @@ static Geometry geometry(int64_t d, int64_t d_block_size, double k_init) {
     return g;
 }
 
-static int fused_check(const ma_tensor *t, const ma_hyper *h) {
+// what every fused route asks of a tensor and the hyper-parameters
+static int common_check(const ma_tensor *t, const ma_hyper *h, Geometry *g) {
     if (!t || !h) return MA_ERR_ARG;
     if (!t->p || !t->g || !t->error || !t->min_vals || !t->max_vals || !t->I || !t->V)
         return MA_ERR_ARG;
@@ -1117,17 +1574,46 @@ static int fused_check(const ma_tensor *t, const ma_hyper *h) {
     if (h->d_block_size < 1 || h->quant_block_size < 1) return MA_ERR_ARG;
     if (!(h->k_init > 0.0 && h->k_init <= 1.0)) return MA_ERR_ARG;
     if (t->index < 0 || t->index >= h->m) return MA_ERR_ARG;
-    const Geometry g = geometry(t->d, h->d_block_size, h->k_init);
-    if (g.dbs > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
-    if (g.k != t->k) return MA_ERR_GEOMETRY;
+    *g = geometry(t->d, h->d_block_size, h->k_init);
+    if (g->dbs > MA_MAX_D_BLOCK) return MA_ERR_BLOCK_SIZE;
+    if (g->k != t->k) return MA_ERR_GEOMETRY;
+    if ((((uintptr_t)t->p | (uintptr_t)t->g) & 15) != 0 || ((uintptr_t)t->error & 3) != 0)
+        return MA_ERR_NOT_FUSABLE;
+    return 0;
+}
+
+static int fused_check(const ma_tensor *t, const ma_hyper *h) {
+    Geometry g;
+    const int rc = common_check(t, h, &g);
+    if (rc) return rc;
     const int64_t q = h->quant_block_size;
     if (q < 8 || q > 512 || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
     if (t->d < q) return MA_ERR_NOT_FUSABLE;
     const bool single = t->d <= h->d_block_size;
     if (!single && (g.dbs % q != 0 || g.dbs % 8 != 0)) return MA_ERR_NOT_FUSABLE;
-    if ((((uintptr_t)t->p | (uintptr_t)t->g) & 15) != 0 || ((uintptr_t)t->error & 3) != 0)
-        return MA_ERR_NOT_FUSABLE;
     return 0;
+}
+
+constexpr int kSpanMaxBlocks = 64;  // top-k blocks one quantisation block may touch
+
+// the three-pass route: alpha > 0, quantisation blocks a multiple of 8 and at least as long
+// as the top-k blocks
+static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
+    Geometry g;
+    const int rc = common_check(t, h, &g);
+    if (rc) return rc;
+    if (!(alpha > 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
+    const int64_t q = h->quant_block_size;
+    if (q % 8 != 0 || q < g.dbs || q >= (1LL << 30)) return MA_ERR_NOT_FUSABLE;
+    if ((q + g.dbs - 1) / g.dbs + 1 > kSpanMaxBlocks) return MA_ERR_NOT_FUSABLE;
+    const bool single = t->d <= h->d_block_size;
+    if (!single && g.dbs % 8 != 0) return MA_ERR_NOT_FUSABLE;
+    return 0;
+}
+
+static inline int64_t span_ws_bytes(const ma_tensor *t, const ma_hyper *h) {
+    const Geometry g = geometry(t->d, h->d_block_size, h->k_init);
+    return (g.n_full + (g.tail > 0 ? 1 : 0)) * 16;  // 2 sets x 4 bf16 words per block
 }
 
 }  // namespace ma
@@ -1323,16 +1809,22 @@ int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
     return fused_check(tensor, hyper);
 }
 
-int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream) {
+static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream,
+                     bool span, double alpha, void *ws, int64_t ws_bytes) {
     if (!tensors || !h || n_tensors < 0) return MA_ERR_ARG;
     for (int i = 0; i < n_tensors; ++i) {
-        const int rc = fused_check(&tensors[i], h);
+        const int rc = span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h);
         if (rc) return rc;
     }
     if (n_tensors == 0) return 0;
+    if (span) {
+        int64_t need = 0;
+        for (int i = 0; i < n_tensors; ++i) need += span_ws_bytes(&tensors[i], h);
+        if (!ws || ws_bytes < need || ((uintptr_t)ws & 7) != 0) return MA_ERR_ARG;
+    }
     hipStream_t s = (hipStream_t)stream;
     int q_shift = 0;
-    while ((1LL << q_shift) < h->quant_block_size) ++q_shift;
+    while (!span && (1LL << q_shift) < h->quant_block_size) ++q_shift;
     WindowWeights W;
     window_weights(h->t, h->m, h->beta1, h->beta2, h->eps, &W);
     const int slot_bytes = h->dtype == MA_BF16 ? 2 : 4;
@@ -1357,18 +1849,32 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
             P.d_block_size = d_block_size;
             P.q_shift = q_shift;
             P.total_items = (int32_t)items;
+            P.q_span = span ? (int32_t)h->quant_block_size : 0;
+            P.alpha = (float)alpha;
+            P.keep = (float)(1.0 - alpha);
             if (P.L.total > kLdsLimit) return MA_ERR_LDS;
-            const int rc = h->dtype == MA_BF16
-                               ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
-                               : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
+            int rc = 0;
+            if (!span) {
+                rc = h->dtype == MA_BF16
+                         ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
+                         : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
+            } else {
+                for (int pass = 1; pass <= 3 && rc == 0; ++pass)
+                    rc = h->dtype == MA_BF16
+                             ? launch_span<RegsBF16>(C, pass, (unsigned)items, P.L.total, s, P)
+                             : launch_span<RegsF32>(C, pass, (unsigned)items, P.L.total, s, P);
+            }
             count = 0;
             items = 0;
             dbs_max = kb_max = 0;
             return rc;
         };
+        int64_t ws_off = 0;
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
             const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
+            const int64_t ws_here = ws_off;
+            if (span) ws_off += span_ws_bytes(&t, h);
             if (chunks_for(g.dbs) != C) continue;
             const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
             if (count == kTensorsPerLaunch || items + nb > 0x7fffffff) {
@@ -1393,6 +1899,7 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
             D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
             D.blk0 = 0;
+            D.ws = span ? reinterpret_cast<uint16_t *>(static_cast<char *>(ws) + ws_here) : nullptr;
             items += nb;
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
@@ -1402,6 +1909,29 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
         if (rc) return rc;
     }
     return 0;
+}
+
+int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream) {
+    return step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0);
+}
+
+int ma_densified_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {
+    return span_check(tensor, hyper, alpha);
+}
+
+int64_t ma_densified_step_workspace(const ma_tensor *tensors, int n_tensors, const ma_hyper *h) {
+    if (!tensors || !h || n_tensors < 0) return -1;
+    int64_t need = 0;
+    for (int i = 0; i < n_tensors; ++i) {
+        if (tensors[i].d <= 0 || h->d_block_size < 1) return -1;
+        need += span_ws_bytes(&tensors[i], h);
+    }
+    return need;
+}
+
+int ma_densified_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, double alpha,
+                      void *workspace, int64_t workspace_bytes, void *stream) {
+    return step_impl(tensors, n_tensors, h, stream, true, alpha, workspace, workspace_bytes);
 }
 
 }  // extern "C"
