@@ -347,7 +347,7 @@ struct TensorDesc {
     float decay;
     int32_t apply_decay;
     int32_t blk0;         // block of the tensor that its first work item stands for
-    uint16_t *ws;         // three-pass route: per-block partial statistics, else unused
+    float *ws;            // two-pass route: per-block extremes of the residual, else unused
 };
 constexpr int kTensorsPerLaunch = 24;
 
@@ -359,7 +359,7 @@ struct FusedParams {
     int32_t d_block_size;
     int32_t q_shift;  // log2(quant_block_size)
     int32_t total_items;  // work items (blocks) of the launch
-    // three-pass route (quantisation blocks at least as long as the top-k blocks)
+    // two-pass route (quantisation blocks at least as long as the top-k blocks)
     int32_t q_span;   // quantisation block length, a multiple of 8
     float alpha;      // share of the dequantised error feedback added to the update
     float keep;       // (float)(1 - alpha): share that stays in the error feedback
@@ -953,16 +953,18 @@ struct FusedBlock {
     }
 
     // =========================================================================================
-    // Three-pass route: quantisation blocks of q_span >= block length elements (q_span a
+    // Two-pass route: quantisation blocks of q_span >= block length elements (q_span a
     // multiple of 8), so a top-k block meets at most two of them and their statistics need
     // every top-k block they cover.  alpha > 0 (MA:296-298, 311-316).
     //   pass 1: a = g + Qinv(e), top-k, window row; the residual r goes to the gradient
-    //           buffer, its min / max per (block, segment) to the workspace (set 0)
-    //   pass 2: e1 = Q(r), d1 = Qinv(e1) in registers; u = Adam(window) + alpha * d1;
-    //           p update; min / max of r2 = (1 - alpha) * d1 to the workspace (set 1)
-    //   pass 3: r2 again from r, e = Q(r2), statistics arrays
+    //           buffer, its exact min / max per (block, segment) to the workspace
+    //   pass 2: statistics of r from the workspace; e1 = Q(r), d1 = Qinv(e1) in registers;
+    //           u = Adam(window) + alpha * d1; p update; r2 = (1 - alpha) * d1; e = Q(r2)
+    // r2 is a non-decreasing function of the code, and the code of the element, so the
+    // statistics of r2 over a quantisation block are r2 at the codes of r's extremes: pass 2
+    // needs no second reduction across blocks.
     // Segment 0 of a block is its part in the quantisation block of its first element,
-    // segment 1 the rest.  Workspace: 4 bf16 words (min0, max0, min1, max1) per block and set.
+    // segment 1 the rest.  Workspace: 4 floats (min0, max0, min1, max1) per block.
     // =========================================================================================
     struct Span {
         int64_t qb0;  // quantisation block of the block's first element
@@ -1006,22 +1008,18 @@ struct FusedBlock {
         }
     }
 
-    __device__ __forceinline__ void store_partials(const BlockGeo &G, int set, float (&mn)[2],
+    __device__ __forceinline__ void store_partials(const BlockGeo &G, float (&mn)[2],
                                                    float (&mx)[2]) {
         wg_minmax2(mn, mx);
-        if (tid == 0) {
-            uint16_t *w = G.D.ws + (block_id(G) * 2 + set) * 4;
-            w[0] = (uint16_t)f2bf(mn[0]);
-            w[1] = (uint16_t)f2bf(mx[0]);
-            w[2] = (uint16_t)f2bf(mn[1]);
-            w[3] = (uint16_t)f2bf(mx[1]);
-        }
+        if (tid == 0)
+            *reinterpret_cast<float4 *>(G.D.ws + block_id(G) * 4) =
+                make_float4(mn[0], mx[0], mn[1], mx[1]);
     }
 
-    // statistics (bf16 bits) of the two quantisation blocks this top-k block meets, from the
+    // exact min / max of r over the two quantisation blocks this top-k block meets, from the
     // partials of all top-k blocks that cover them (at most 64 each: lane i takes one)
-    __device__ __forceinline__ void gather_stats(const BlockGeo &G, const Span &S, int set,
-                                                 uint32_t (&mnb)[2], uint32_t (&mxb)[2]) const {
+    __device__ __forceinline__ void gather_extremes(const BlockGeo &G, const Span &S,
+                                                    float (&mnx)[2], float (&mxx)[2]) const {
         const int64_t q = P.q_span;
         const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
         const int64_t nblk = (G.D.d + dbs - 1) / dbs;
@@ -1037,14 +1035,39 @@ struct FusedBlock {
                 const int64_t b = b_lo + lane;
                 if (b <= b_hi) {
                     const int seg = b * dbs >= first ? 0 : 1;
-                    const uint16_t *w = G.D.ws + (b * 2 + set) * 4 + seg * 2;
-                    mn = bf2f(w[0]);
-                    mx = bf2f(w[1]);
+                    const float *w = G.D.ws + b * 4 + seg * 2;
+                    mn = w[0];
+                    mx = w[1];
                 }
                 group_minmax<0>(mn, mx, kWave);
             }
-            mnb[s2] = f2bf(mn);
-            mxb[s2] = f2bf(mx);
+            mnx[s2] = mn;
+            mxx[s2] = mx;
+        }
+    }
+
+    // Statistics of r (sp_mn / sp_mx) and of r2 (sp2_mn / sp2_mx) for both segments, from the
+    // exact extremes of r.
+    __device__ __forceinline__ void span_statistics(const BlockGeo &G, const Span &S) {
+        float mnx[2], mxx[2];
+        gather_extremes(G, S, mnx, mxx);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            sp_mn[s2] = f2bf(mnx[s2]);
+            sp_mx[s2] = f2bf(mxx[s2]);
+            const float mnf = bf2f(sp_mn[s2]);
+            const float u = div15(bf2f(sp_mx[s2]) - mnf, d15);
+            float x[8], cf[8];
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) x[e] = (e & 1) ? mxx[s2] : mnx[s2];
+            codes8(x, mnf, u, cf);
+            float lo = cf[0] * u, hi = cf[1] * u;
+            lo = lo + mnf;
+            hi = hi + mnf;
+            lo = P.keep * lo;
+            hi = P.keep * hi;
+            sp2_mn[s2] = f2bf(to_elem(0.0f + lo));
+            sp2_mx[s2] = f2bf(to_elem(0.0f + hi));
         }
     }
 
@@ -1098,7 +1121,8 @@ struct FusedBlock {
     }
 
     // ---- pass 1 ------------------------------------------------------------------------------
-    uint32_t sp_mn[2], sp_mx[2];  // statistics of the two segments (bf16 bits), wave-uniform
+    uint32_t sp_mn[2], sp_mx[2];    // statistics of r in the two segments (bf16 bits)
+    uint32_t sp2_mn[2], sp2_mx[2];  // statistics of r2
 
     __device__ __forceinline__ void span_load_grad_inputs(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
@@ -1184,10 +1208,10 @@ struct FusedBlock {
                 store8(out, off, FULL ? 0x7fffffff : n, true, x);
             }
         }
-        store_partials(G, 0, mn, mx);
+        store_partials(G, mn, mx);
     }
 
-    // ---- pass 2 and 3 -----------------------------------------------------------------------
+    // ---- pass 2 -----------------------------------------------------------------------
     __device__ __forceinline__ void span_load_residual(const BlockGeo &G) {
         const int n = FULL ? C * kRound : G.n;
         const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
@@ -1207,17 +1231,19 @@ struct FusedBlock {
         }
     }
 
-    // p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u; partial statistics of
-    // r2 = rne(0 + keep * d1).  After window_stage.
+    // p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u; r2 = rne(0 + keep * d1);
+    // e = Q(r2); statistics arrays.  After window_stage.
     __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        uint8_t *err = D.err + (G.e0 >> 1);
         const float neg_lr = D.neg_lr, decay = D.decay;
         const bool apply_decay = D.apply_decay != 0;
         const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
         const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
-        float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+        const float m20 = bf2f(sp2_mn[0]), m21 = bf2f(sp2_mn[1]);
+        const float v0 = div15(bf2f(sp2_mx[0]) - m20, d15), v1 = div15(bf2f(sp2_mx[1]) - m21, d15);
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -1243,7 +1269,7 @@ struct FusedBlock {
                     uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
                     uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
                 }
-                float lmn = INFINITY, lmx = -INFINITY;
+                float r2[8], cf[8];
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
                     if (apply_decay) pv[e] = to_elem(pv[e] * decay);
@@ -1252,45 +1278,9 @@ struct FusedBlock {
                     const float prod = neg_lr * ud;
                     pv[e] = pv[e] + prod;
                     const float keep = P.keep * d1[e];
-                    const float r2 = to_elem(0.0f + keep);
-                    if (FULL || off + e < n) {
-                        lmn = fmin_raw(lmn, r2);
-                        lmx = fmax_raw(lmx, r2);
-                    }
-                }
-                mn[0] = fmin_raw(mn[0], second ? INFINITY : lmn);
-                mx[0] = fmax_raw(mx[0], second ? -INFINITY : lmx);
-                mn[1] = fmin_raw(mn[1], second ? lmn : INFINITY);
-                mx[1] = fmax_raw(mx[1], second ? lmx : -INFINITY);
-                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        store_partials(G, 1, mn, mx);
-    }
-
-    // e = Q(r2) against the statistics of r2, and the statistics arrays themselves
-    __device__ __forceinline__ void span_final_codes(const BlockGeo &G, const Span &S,
-                                                     const uint32_t (&mn2b)[2],
-                                                     const uint32_t (&mx2b)[2]) {
-        const int n = FULL ? C * kRound : G.n;
-        uint8_t *err = G.D.err + (G.e0 >> 1);
-        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
-        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
-        const float m20 = bf2f(mn2b[0]), m21 = bf2f(mn2b[1]);
-        const float v0 = div15(bf2f(mx2b[0]) - m20, d15), v1 = div15(bf2f(mx2b[1]) - m21, d15);
-#pragma unroll
-        for (int c = 0; c < C; ++c) {
-            const int off = chunk_off<C>(wave, c, lane);
-            if (FULL || off < n) {
-                const bool second = off >= S.bnd;
-                float d1[8], r2[8], cf[8];
-                span_requant(c, second ? mn1 : mn0, second ? u1 : u0, d1);
-#pragma unroll
-                for (int e = 0; e < kChunk; ++e) {
-                    const float keep = P.keep * d1[e];
                     r2[e] = to_elem(0.0f + keep);
                 }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
                 codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
@@ -1309,12 +1299,12 @@ struct FusedBlock {
         // the block that holds the first element of a quantisation block writes its statistics
         if (tid == 0) {
             if (G.e0 == S.qb0 * (int64_t)P.q_span) {
-                G.D.mn[S.qb0] = (uint16_t)mn2b[0];
-                G.D.mx[S.qb0] = (uint16_t)mx2b[0];
+                D.mn[S.qb0] = (uint16_t)sp2_mn[0];
+                D.mx[S.qb0] = (uint16_t)sp2_mx[0];
             }
             if (S.bnd != 0x7fffffff) {
-                G.D.mn[S.qb0 + 1] = (uint16_t)mn2b[1];
-                G.D.mx[S.qb0 + 1] = (uint16_t)mx2b[1];
+                D.mn[S.qb0 + 1] = (uint16_t)sp2_mn[1];
+                D.mx[S.qb0 + 1] = (uint16_t)sp2_mx[1];
             }
         }
     }
@@ -1362,7 +1352,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     }
 }
 
-// Three-pass route, see FusedBlock.  PASS 1 / 2 / 3; one workgroup per block.
+// Two-pass route, see FusedBlock.  PASS 1 / 2; one workgroup per block.
 template <class R, int MIN_WAVES, int PASS>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -1375,19 +1365,13 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             fb.span_dequant(G, S);
             fb.topk_and_row(G);
             fb.span_store_residual(G, S);
-        } else if constexpr (PASS == 2) {
+        } else {
             fb.row_in_lds = false;
             fb.load_params_window(G);
             fb.span_load_residual(G);
-            fb.gather_stats(G, S, 0, fb.sp_mn, fb.sp_mx);
+            fb.span_statistics(G, S);
             fb.window_stage(G);
             fb.span_param_stage(G, S);
-        } else {
-            fb.span_load_residual(G);
-            fb.gather_stats(G, S, 0, fb.sp_mn, fb.sp_mx);
-            uint32_t mn2[2], mx2[2];
-            fb.gather_stats(G, S, 1, mn2, mx2);
-            fb.span_final_codes(G, S, mn2, mx2);
         }
     };
     if (G.n == R::kC * kRound) {
@@ -1518,20 +1502,14 @@ template <class R>
 static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
                            const FusedParams &P) {
     int rc;
-    switch (pass) {
-        case 1:
-            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
-            if (rc) return rc;
-            span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
-            break;
-        case 2:
-            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
-            if (rc) return rc;
-            span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
-            break;
-        default:
-            span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
-            break;
+    if (pass == 1) {
+        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
+        if (rc) return rc;
+        span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
+    } else {
+        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
+        if (rc) return rc;
+        span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
     }
     return launch_status();
 }
@@ -1596,7 +1574,7 @@ static int fused_check(const ma_tensor *t, const ma_hyper *h) {
 
 constexpr int kSpanMaxBlocks = 64;  // top-k blocks one quantisation block may touch
 
-// the three-pass route: alpha > 0, quantisation blocks a multiple of 8 and at least as long
+// the two-pass route: 0 < alpha < 1, quantisation blocks a multiple of 8 and at least as long
 // as the top-k blocks
 static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
     Geometry g;
@@ -1613,7 +1591,7 @@ static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
 
 static inline int64_t span_ws_bytes(const ma_tensor *t, const ma_hyper *h) {
     const Geometry g = geometry(t->d, h->d_block_size, h->k_init);
-    return (g.n_full + (g.tail > 0 ? 1 : 0)) * 16;  // 2 sets x 4 bf16 words per block
+    return (g.n_full + (g.tail > 0 ? 1 : 0)) * 16;  // 4 floats per block
 }
 
 }  // namespace ma
@@ -1820,7 +1798,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     if (span) {
         int64_t need = 0;
         for (int i = 0; i < n_tensors; ++i) need += span_ws_bytes(&tensors[i], h);
-        if (!ws || ws_bytes < need || ((uintptr_t)ws & 7) != 0) return MA_ERR_ARG;
+        if (!ws || ws_bytes < need || ((uintptr_t)ws & 15) != 0) return MA_ERR_ARG;
     }
     hipStream_t s = (hipStream_t)stream;
     int q_shift = 0;
@@ -1859,7 +1837,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                          ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
                          : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
             } else {
-                for (int pass = 1; pass <= 3 && rc == 0; ++pass)
+                for (int pass = 1; pass <= 2 && rc == 0; ++pass)
                     rc = h->dtype == MA_BF16
                              ? launch_span<RegsBF16>(C, pass, (unsigned)items, P.L.total, s, P)
                              : launch_span<RegsF32>(C, pass, (unsigned)items, P.L.total, s, P);
@@ -1899,7 +1877,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
             D.blk0 = 0;
-            D.ws = span ? reinterpret_cast<uint16_t *>(static_cast<char *>(ws) + ws_here) : nullptr;
+            D.ws = span ? reinterpret_cast<float *>(static_cast<char *>(ws) + ws_here) : nullptr;
             items += nb;
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
