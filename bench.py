@@ -137,6 +137,17 @@ def cpu_baseline(workload, budget_s=20.0):
                       f"{steps} steps, C oracle with OpenMP"}
 
 
+def route_label(opt, params):
+    """Which route the optimizer takes for the tensors of the list, e.g. "fused" or
+    "densified" when all go one way, else counts per route."""
+    names = {0: "op-by-op", 1: "fused", 2: "densified"}
+    counts = {}
+    for p in params:
+        r = opt._fusable(p, opt.state[p]) if opt.use_fused else 0
+        counts[names[r]] = counts.get(names[r], 0) + 1
+    return next(iter(counts)) if len(counts) == 1 else counts
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,7 +240,7 @@ def main():
                    "tensors": len(shapes), "m": m,
                    "k_init": k_init, "quant_block_size": q, "alpha": alpha,
                    "d_block_size": opt.d_block_size,
-                   "route": "op-by-op" if args.op_by_op else "fused"},
+                   "route": route_label(opt, params)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op)),

@@ -73,3 +73,29 @@ def test_fused_step_check_rejects_bad_layouts():
     t.g = 0x10000
     h.m = 65
     assert chk() == -3
+
+
+def test_densified_step_check_and_workspace():
+    """Host-only validation of ma_densified_step's conditions and its workspace size."""
+    from ista_daslab_optimizers import _hip
+    t = _hip.MaTensor()
+    for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
+        setattr(t, f, 0x10000)
+    t.d, t.k, t.lr, t.weight_decay, t.index = 20480 * 2 + 4096, 205 * 2 + 41, 1e-3, 0.0, 0
+    h = _hip.MaHyper(1, 10, _hip.MA_BF16, 100000, 20480, 0.01, 0.9, 0.999, 1e-8)
+    chk = lambda a: _hip.lib.ma_densified_step_check(ctypes.byref(t), ctypes.byref(h), a)
+    assert chk(0.5) == 0
+    assert chk(0.0) == _hip.MA_ERR_NOT_FUSABLE      # alpha == 0 is ma_fused_step's case
+    assert chk(1.0) == _hip.MA_ERR_NOT_FUSABLE      # micro_adam.py:18 asks for alpha < 1
+    h.quant_block_size = 100001                     # not a multiple of 8
+    assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
+    h.quant_block_size = 64                         # shorter than the top-k block
+    assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
+    h.quant_block_size = 20480 * 100                # covers more top-k blocks than one wave reads
+    assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
+    h.quant_block_size = 100000
+    arr = (_hip.MaTensor * 2)(t, t)
+    assert _hip.lib.ma_densified_step_workspace(arr, 2, ctypes.byref(h)) == 2 * 3 * 16
+    # too small a workspace is refused before anything is launched
+    rc = _hip.lib.ma_densified_step(arr, 2, ctypes.byref(h), 0.5, 0x10000, 16, None)
+    assert rc == -1  # MA_ERR_ARG

@@ -117,3 +117,33 @@ def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, step
                 touched[(torch.arange(k, device="cuda") // km) * dbs + sa["I"][r].long()] = True
             moved = (p.data.view(-1) != p0.view(-1))
             assert not bool((moved & ~touched).any())
+
+
+def test_densified_and_opbyop_agree_at_llama3_shapes():
+    """alpha = 0.5 with quantisation blocks of 100000 elements (they straddle the 20480-element
+    top-k blocks): the two-pass fused route and the op-by-op kernels, which form the statistics
+    in different ways, end in bit-identical parameters and state."""
+    from ista_daslab_optimizers import MicroAdam
+    shapes = [(14336, 4096), (1024, 4096), (4096,)]
+    dtype = torch.bfloat16
+    torch.manual_seed(0)
+    pa = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in shapes]
+    pb = [torch.nn.Parameter(p.detach().clone()) for p in pa]
+    kw = dict(m=10, lr=1e-3, quant_block_size=100000, k_init=0.01, alpha=0.5)
+    oa, ob = MicroAdam(pa, **kw), MicroAdam(pb, **kw)
+    ob.use_fused = False
+    for step in range(12):
+        grads = [_grads(s, "normal", step * 10 + i, dtype) for i, s in enumerate(shapes)]
+        for p, p2, g in zip(pa, pb, grads):
+            p.grad, p2.grad = g.clone(), g.clone()
+        oa.step()
+        ob.step()
+        for p, p2 in zip(pa, pb):
+            sa, sb = oa.state[p], ob.state[p2]
+            assert oa._fusable(p, sa) == 2 and sa["index"] == sb["index"]
+            assert torch.equal(p.data, p2.data), f"step {step}: parameters differ between routes"
+            for key in ("error", "min_vals", "max_vals"):
+                assert torch.equal(sa[key], sb[key]), (step, key)
+            Ia, Va = _canon(sa["I"], sa["V"], sa["k_block_size_many"])
+            Ib, Vb = _canon(sb["I"], sb["V"], sb["k_block_size_many"])
+            assert torch.equal(Ia, Ib) and torch.equal(Va, Vb), (step, "window")
