@@ -695,13 +695,13 @@ __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, 
 
 // ---- Adam statistics of one block from its window rows ---------------------------------------------
 //
-// slot[i] (one cell per block coordinate, zeroed by the caller) maps a coordinate to 1 + its
-// row in z1 / z2 / coord; rows are handed out on first touch.  Only coordinates in [lo, hi) are
-// considered, so a caller short of LDS can walk the block in several ranges.  Window rows are
-// visited in increasing row order with a barrier between rows, and inside a row all indices are
-// distinct, so every coordinate's sums are formed in a fixed order.  On return (after a
-// barrier) `*counter` holds the number of touched coordinates (at most `cap`), coord[s] their
-// block-relative index and z1[s], z2[s] the weighted sums.
+// General form, for windows too large for the one-pass stage of the fused kernel: the block is
+// walked in coordinate ranges [lo, hi) short enough for two dense fp32 arrays z1 / z2 in LDS
+// (one cell per coordinate of the range).  Window rows are visited in increasing row order with
+// a barrier between rows, and inside a row all indices are distinct, so every coordinate's sums
+// are formed in a fixed order.  The entries are fetched kWindowDepth steps ahead of their use.
+// On return (after a barrier) z1[c - lo], z2[c - lo] hold the weighted sums of coordinate c, both
+// zero where no row names it.
 struct WindowView {
     const int16_t *I;   // window indices, row stride k, already offset to this block's columns
     const uint16_t *V;  // window values, same layout
@@ -714,73 +714,67 @@ struct WindowView {
     const float *w2;
 };
 
-// One window entry per thread: add (w1*v, w2*v*v) to the sums of coordinate idx, handing out
-// a fresh row of z1 / z2 / coord when the coordinate is seen for the first time.  Must be
-// called by every lane of the wave (inactive lanes pass active = false).
-template <typename slot_t>
-__device__ __forceinline__ void window_entry(int idx, uint32_t vb, bool active, float w1,
-                                             float w2, slot_t *slot, float *z1, float *z2,
-                                             uint16_t *coord, uint32_t *counter, int cap,
-                                             int lane) {
-    const float v = bf2f(vb);
-    const float a1 = w1 * v;
-    const float vv = v * v;
-    const float a2 = w2 * vv;
-    uint32_t s = active ? (uint32_t)slot[idx] : 1u;
-    const bool fresh = active && s == 0;
-    const uint64_t mask = __ballot(fresh);
-    if (mask != 0) {
-        const int leader = __ffsll((unsigned long long)mask) - 1;
-        uint32_t first = 0;
-        if (lane == leader) first = atomicAdd(counter, (uint32_t)__popcll(mask));
-        first = __shfl(first, leader, kWave);
-        if (fresh) {
-            s = first + mbcnt(mask) + 1;
-            if (s <= (uint32_t)cap) {  // always true for duplicate-free rows
-                slot[idx] = (slot_t)s;
-                coord[s - 1] = (uint16_t)idx;
-                z1[s - 1] = 0.0f + a1;
-                z2[s - 1] = 0.0f + a2;
-            }
-        }
-    }
-    if (active && !fresh) {
-        z1[s - 1] = z1[s - 1] + a1;
-        z2[s - 1] = z2[s - 1] + a2;
-    }
-}
+constexpr int kWindowDepth = 8;
 
-template <typename slot_t>
 __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, int lo, int hi,
-                                                  slot_t *slot, float *z1, float *z2,
-                                                  uint16_t *coord, uint32_t *counter, int cap) {
-    const int tid = opaque_tid(), lane = tid & 63;
-    if (tid == 0) *counter = 0;
+                                                  float *z1, float *z2) {
+    const int tid = opaque_tid();
+    for (int i = tid; i < hi - lo; i += kWG) {
+        z1[i] = 0.0f;
+        z2[i] = 0.0f;
+    }
     __syncthreads();
     const int trips = (kb + kWG - 1) / kWG;
-    for (int row = 0; row < wv.rows; ++row) {
-        const float w1 = wv.w1[row], w2 = wv.w2[row];
-        for (int it = 0; it < trips; ++it) {
-            const int j = it * kWG + tid;
-            int idx = 0;
-            uint32_t vb = 0;
-            bool active = j < kb;
-            if (active) {
+    const int steps = wv.rows * trips;
+    // step s is entry j = (s % trips) * kWG + tid of row s / trips; idx 0xffff: nothing
+    auto fetch = [&](int s, uint32_t &idx, uint32_t &vb) {
+        idx = 0xffffu;
+        vb = 0;
+        if (s < steps) {
+            const int row = s / trips;
+            const int j = (s - row * trips) * kWG + tid;
+            if (j < kb) {
                 if (row == wv.cur_row) {
                     idx = wv.cur_idx[j];
                     vb = wv.cur_val[j];
                 } else {
-                    idx = wv.I[(int64_t)row * wv.k + j];
+                    idx = (uint16_t)wv.I[(int64_t)row * wv.k + j];
                     vb = wv.V[(int64_t)row * wv.k + j];
                 }
-                // the range test also keeps a corrupt index from leaving the block; +-0 values
-                // add nothing and are skipped, which keeps the all-(0, 0) rows of a fresh
-                // window from naming coordinate 0 many times in one row
-                active = idx >= lo && idx < hi && (vb & 0x7fffu) != 0;
             }
-            window_entry(idx, vb, active, w1, w2, slot, z1, z2, coord, counter, cap, lane);
         }
-        __syncthreads();
+    };
+    uint32_t nI[kWindowDepth], nV[kWindowDepth];
+#pragma unroll
+    for (int i = 0; i < kWindowDepth; ++i) fetch(i, nI[i], nV[i]);
+    for (int base = 0; base < steps; base += kWindowDepth) {
+        uint32_t cI[kWindowDepth], cV[kWindowDepth];
+#pragma unroll
+        for (int i = 0; i < kWindowDepth; ++i) {
+            cI[i] = nI[i];
+            cV[i] = nV[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kWindowDepth; ++i) fetch(base + kWindowDepth + i, nI[i], nV[i]);
+#pragma unroll
+        for (int i = 0; i < kWindowDepth; ++i) {
+            const int s = base + i;
+            if (s < steps) {
+                const int row = s / trips;
+                const int idx = (int)cI[i];
+                // the range test also keeps a corrupt index from leaving the block; +-0 values
+                // add nothing and are skipped (the rows of a fresh window are all (0, 0))
+                if (idx >= lo && idx < hi && (cV[i] & 0x7fffu) != 0) {
+                    const float v = bf2f(cV[i]);
+                    const float a1 = wv.w1[row] * v;
+                    const float vv = v * v;
+                    const float a2 = wv.w2[row] * vv;
+                    z1[idx - lo] = z1[idx - lo] + a1;
+                    z2[idx - lo] = z2[idx - lo] + a2;
+                }
+                if (s - row * trips == trips - 1) __syncthreads();
+            }
+        }
     }
 }
 

@@ -293,12 +293,8 @@ __global__ __launch_bounds__(kWG) void window_update_kernel(int64_t d, int dbs, 
                                                             const uint16_t *V, T *out,
                                                             WindowWeights W, LdsMap L) {
     extern __shared__ __align__(16) unsigned char lds[];
-    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
-    uint32_t *counter = sh + kShCounter;
-    uint16_t *slot = reinterpret_cast<uint16_t *>(lds + L.off_slot);
     float *z1 = reinterpret_cast<float *>(lds + L.off_union);
     float *z2 = z1 + L.z_cap;
-    uint16_t *coord = reinterpret_cast<uint16_t *>(z2 + L.z_cap);
     const int tid = threadIdx.x;
     const int64_t b = blockIdx.x;
     const int64_t e0 = b * dbs;
@@ -316,13 +312,12 @@ __global__ __launch_bounds__(kWG) void window_update_kernel(int64_t d, int dbs, 
     wv.cur_val = nullptr;
     wv.w1 = W.w1;
     wv.w2 = W.w2;
-    for (int i = tid; i < L.slot_cells; i += kWG) slot[i] = 0;
     for (int lo = 0; lo < n; lo += L.sub_len) {
         const int hi = lo + L.sub_len < n ? lo + L.sub_len : n;
-        window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, L.z_cap);
-        const int cnt = (int)(*counter < (uint32_t)L.z_cap ? *counter : (uint32_t)L.z_cap);
-        for (int s = tid; s < cnt; s += kWG)
-            stf(out, e0 + coord[s], adam_direction(z1[s], z2[s], W.s1, W.s2, W.eps));
+        window_accumulate(wv, kb, lo, hi, z1, z2);
+        for (int c = tid; c < hi - lo; c += kWG)
+            if (z1[c] != 0.0f || z2[c] != 0.0f)
+                stf(out, e0 + lo + c, adam_direction(z1[c], z2[c], W.s1, W.s2, W.eps));
         __syncthreads();
     }
 }
@@ -892,12 +887,12 @@ struct FusedBlock {
             wv.w2 = P.W.w2;
             for (int lo = 0; lo < n; lo += P.L.sub_len) {
                 const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
-                window_accumulate(wv, kb, lo, hi, slot, z1, z2, coord, counter, P.L.z_cap);
-                const int cnt =
-                    (int)(*counter < (uint32_t)P.L.z_cap ? *counter : (uint32_t)P.L.z_cap);
-                for (int s = tid; s < cnt; s += kWG) {
-                    const float u = adam_direction(z1[s], z2[s], P.W.s1, P.W.s2, P.W.eps);
-                    slot[coord[s]] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                window_accumulate(wv, kb, lo, hi, z1, z2);
+                for (int c = tid; c < hi - lo; c += kWG) {
+                    if (z1[c] != 0.0f || z2[c] != 0.0f) {
+                        const float u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                        slot[lo + c] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                    }
                 }
                 __syncthreads();
             }
@@ -1391,25 +1386,25 @@ static inline int align16(int x) { return (x + 15) & ~15; }
 
 // LDS plan for a block kernel: longest block `dbs_max`, most entries per block row `kb_max`,
 // window length m, bytes per slot cell.
-static LdsMap plan_lds(int dbs_max, int kb_max, int m, int slot_bytes) {
+static LdsMap plan_lds(int dbs_max, int kb_max, int m, int slot_bytes, bool one_pass = true) {
     LdsMap L;
     L.off_sel_idx = kMiscBytes;
     L.off_sel_val = L.off_sel_idx + align16(kb_max * 2);
     L.off_slot = L.off_sel_val + align16(kb_max * 2);
     L.slot_cells = (dbs_max + 7) & ~7;
     L.off_union = L.off_slot + align16(L.slot_cells * slot_bytes);
+    // one-pass window stage: two floats and four 16-bit words per entry; otherwise the block is
+    // walked in coordinate ranges of at most 4096 with two dense fp32 arrays
     const int64_t entries = (int64_t)m * kb_max;
-    if (entries <= 4096) {
-        L.sub_len = L.slot_cells;
-        L.z_cap = (int)(entries < 8 ? 8 : entries);
-    } else {
-        L.sub_len = 4096;
-        L.z_cap = 4096;
-    }
-    // one-pass window stage: two floats and four 16-bit words per entry
     L.fast_cap = 0;
-    if (entries <= kEnt * kWG && m <= kFastRows) L.fast_cap = L.z_cap;
-    const int zbytes = L.z_cap * (L.fast_cap ? 16 : 10);
+    if (one_pass && entries <= kEnt * kWG && m <= kFastRows) {
+        L.fast_cap = L.z_cap = (int)(entries < 8 ? 8 : entries);
+        L.sub_len = L.slot_cells;
+    } else {
+        L.sub_len = L.slot_cells < 4096 ? L.slot_cells : 4096;
+        L.z_cap = L.sub_len;
+    }
+    const int zbytes = L.z_cap * (L.fast_cap ? 16 : 8);
     L.total = L.off_union + align16(zbytes > kHistBytes ? zbytes : kHistBytes);
     return L;
 }
@@ -1761,7 +1756,7 @@ int ma_compute_microadam_update(int blocks, int threads, int carveout, int64_t t
     if ((nblocks - 1) * d_block_size >= d) return MA_ERR_GEOMETRY;
     WindowWeights W;
     window_weights(t, (int)m, beta1, beta2, eps, &W);
-    const LdsMap L = plan_lds((int)d_block_size, (int)k_block_size, (int)m, 2);
+    const LdsMap L = plan_lds((int)d_block_size, (int)k_block_size, (int)m, 2, false);
     if (L.total > kLdsLimit) return MA_ERR_LDS;
     hipStream_t s = (hipStream_t)stream;
     int rc;
