@@ -152,7 +152,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps; default m + 2, so that the window is full when timing starts")
     ap.add_argument("--workload", default="llama2-7b", choices=sorted(WORKLOADS))
     ap.add_argument("--grad-sets", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -168,6 +169,8 @@ def main():
     from ista_daslab_optimizers import MicroAdam
 
     shapes_fn, dtype, m, k_init, q, alpha, gstd = WORKLOADS[args.workload]
+    if args.warmup is None:
+        args.warmup = m + 2
     shapes = shapes_fn()
     tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
     dev = torch.device("cuda:0")

@@ -726,27 +726,36 @@ __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, 
     __syncthreads();
     const int trips = (kb + kWG - 1) / kWG;
     const int steps = wv.rows * trips;
-    // step s is entry j = (s % trips) * kWG + tid of row s / trips; idx 0xffff: nothing
-    auto fetch = [&](int s, uint32_t &idx, uint32_t &vb) {
-        idx = 0xffffu;
+    // Step s is entry j = it * kWG + tid of window row `row`, (row, it) counting up with `it`
+    // the faster digit; the fetch stream runs kWindowDepth steps ahead of the process stream.
+    int frow = 0, fit = 0;  // wave-uniform
+    auto fetch = [&](uint32_t &idx, uint32_t &vb) {
+        idx = 0xffffu;  // never inside a range
         vb = 0;
-        if (s < steps) {
-            const int row = s / trips;
-            const int j = (s - row * trips) * kWG + tid;
+        if (frow < wv.rows) {
+            const int j = fit * kWG + tid;
             if (j < kb) {
-                if (row == wv.cur_row) {
+                if (frow == wv.cur_row) {
                     idx = wv.cur_idx[j];
                     vb = wv.cur_val[j];
                 } else {
-                    idx = (uint16_t)wv.I[(int64_t)row * wv.k + j];
-                    vb = wv.V[(int64_t)row * wv.k + j];
+                    const int16_t *Ir = wv.I + (int64_t)frow * wv.k;
+                    const uint16_t *Vr = wv.V + (int64_t)frow * wv.k;
+                    idx = (uint16_t)Ir[j];
+                    vb = Vr[j];
                 }
+            }
+            if (++fit == trips) {
+                fit = 0;
+                ++frow;
             }
         }
     };
     uint32_t nI[kWindowDepth], nV[kWindowDepth];
 #pragma unroll
-    for (int i = 0; i < kWindowDepth; ++i) fetch(i, nI[i], nV[i]);
+    for (int i = 0; i < kWindowDepth; ++i) fetch(nI[i], nV[i]);
+    int prow = 0, pit = 0;
+    const uint32_t span = (uint32_t)(hi - lo);
     for (int base = 0; base < steps; base += kWindowDepth) {
         uint32_t cI[kWindowDepth], cV[kWindowDepth];
 #pragma unroll
@@ -755,24 +764,26 @@ __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, 
             cV[i] = nV[i];
         }
 #pragma unroll
-        for (int i = 0; i < kWindowDepth; ++i) fetch(base + kWindowDepth + i, nI[i], nV[i]);
+        for (int i = 0; i < kWindowDepth; ++i) fetch(nI[i], nV[i]);
 #pragma unroll
         for (int i = 0; i < kWindowDepth; ++i) {
-            const int s = base + i;
-            if (s < steps) {
-                const int row = s / trips;
-                const int idx = (int)cI[i];
+            if (prow < wv.rows) {
+                const uint32_t c = cI[i] - (uint32_t)lo;
                 // the range test also keeps a corrupt index from leaving the block; +-0 values
                 // add nothing and are skipped (the rows of a fresh window are all (0, 0))
-                if (idx >= lo && idx < hi && (cV[i] & 0x7fffu) != 0) {
+                if (c < span && (cV[i] & 0x7fffu) != 0) {
                     const float v = bf2f(cV[i]);
-                    const float a1 = wv.w1[row] * v;
+                    const float a1 = wv.w1[prow] * v;
                     const float vv = v * v;
-                    const float a2 = wv.w2[row] * vv;
-                    z1[idx - lo] = z1[idx - lo] + a1;
-                    z2[idx - lo] = z2[idx - lo] + a2;
+                    const float a2 = wv.w2[prow] * vv;
+                    z1[c] = z1[c] + a1;
+                    z2[c] = z2[c] + a2;
                 }
-                if (s - row * trips == trips - 1) __syncthreads();
+                if (++pit == trips) {
+                    pit = 0;
+                    ++prow;
+                    __syncthreads();
+                }
             }
         }
     }
