@@ -388,14 +388,14 @@ typedef struct {
     double lr, wd;
 } ora_hyper;
 
-/* micro_adam.py:146-328 for alpha in [0, 1).  `grad` is consumed as scratch, as in
+/* micro_adam.py:146-328 for alpha in [0, 1) and alpha == -2.  `grad` is consumed as scratch, as in
  * the reference (:153).  `index` is the ring position (:180, :211) and is
- * advanced.  Returns 0, or -1 for the unsupported alpha == -2 mode. */
+ * advanced.  Returns 0, or -1 for any other alpha. */
 int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d, int64_t *index,
                     int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
                     uint16_t *max_vals) {
     ora_geom g;
-    if (h->alpha < 0) return -1;
+    if (h->alpha < 0 && h->alpha != -2.0) return -1;
     ora_geometry(d, h->max_d_block_size, h->k_init, h->q, &g);
     int64_t row = *index;
     int16_t *I_row = I + row * g.k;
@@ -417,6 +417,15 @@ int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t 
     ora_asymm_block_quant(d, h->q, error, min_vals, max_vals, grad, dtype);
     /* :234-235 */
     if (h->wd > 0) ora_weight_decay(d, p, (float)(1.0 - h->lr * h->wd), dtype);
+    /* :238-273, alpha == -2: p = p - a + Qinv(e_new).  The quant_err vector of :259-261, :271
+     * only feeds the logged norms. */
+    if (h->alpha == -2.0) {
+        ora_param_update(d, p, grad, -1.0f, dtype, dtype);                       /* STEP A, :264 */
+        if (dtype == ORA_BF16) memset(grad, 0, (size_t)d * 2);                   /* :267 */
+        else memset(grad, 0, (size_t)d * 4);
+        ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad, 1.0f, dtype);
+        ora_param_update(d, p, grad, 1.0f, dtype, dtype);                        /* STEP B, :269 */
+    }
     /* STEPS 10-11, :276-291 */
     if (dtype == ORA_BF16) memset(grad, 0, (size_t)d * 2);
     else memset(grad, 0, (size_t)d * 4);

@@ -249,5 +249,5 @@ class OracleMicroAdam:
                                        _ptr(st["error"]), _ptr(st["min_vals"]),
                                        _ptr(st["max_vals"]))
             if rc != 0:
-                raise NotImplementedError("oracle covers alpha in [0, 1)")
+                raise NotImplementedError("oracle covers alpha in [0, 1) and alpha == -2")
             st["index"] = idx.value

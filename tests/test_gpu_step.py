@@ -80,6 +80,9 @@ GENERAL_CASES = [
     ([999], torch.float32, 2, 100, 0.03, 0.25, 0.01, 400, 5),
     ([20480 * 3 + 77], torch.bfloat16, 4, 100001, 0.01, 0.5, 0.0, 20480, 6),
     ([50, 20], torch.bfloat16, 3, 64, 0.1, 0.0, 0.0, 20480, 4),
+    # alpha == -2: the quantisation error goes straight into the parameters (micro_adam.py:238-273)
+    ([20480 + 4096, 300], torch.bfloat16, 4, 64, 0.01, -2, 0.0, 20480, 6),
+    ([3000], torch.float32, 3, 64, 0.02, -2, 0.05, 1024, 5),
 ]
 
 

@@ -399,6 +399,8 @@ CASES = [
     ([2500, 130], torch.bfloat16, 5, 32, 0.05, 0.0, 0.1, 512, 8),
     ([4100, 33], torch.bfloat16, 3, 1000, 0.01, 0.5, 0.0, 1024, 7),
     ([999], torch.float32, 2, 100, 0.03, 0.25, 0.01, 400, 5),
+    ([3000, 257], torch.bfloat16, 4, 64, 0.01, -2, 0.0, 1024, 6),     # micro_adam.py:238-273
+    ([1500], torch.float32, 3, 64, 0.02, -2, 0.05, 512, 5),
 ]
 
 

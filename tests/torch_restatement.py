@@ -153,6 +153,12 @@ class TorchMicroAdam:
             quantize(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad)
             if self.wd > 0:
                 p.mul_(1 - lr * self.wd)
+            if self.alpha == -2:
+                # micro_adam.py:264-269: p = p - a, then p = p + Qinv(e_new)
+                p.add_(grad, alpha=-1)
+                grad.zero_()
+                qinv_accumulate(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad, 1.0)
+                p.add_(grad)
             grad.zero_()
             self._adam_direction(st, grad, d)
             if self.alpha > 0:
