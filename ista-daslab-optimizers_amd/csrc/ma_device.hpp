@@ -551,45 +551,40 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         ok = ok && cnts[w] <= (uint32_t)kCandPerWave;
     }
     if (ok) {
-        // Exact top-kb among the candidates (at most two per thread): a radix select on their
-        // keys gives the threshold key T and the number of entries equal to T to keep; entries
-        // above T get consecutive output slots by a prefix sum over the threads, entries equal
-        // to T are ranked among themselves by index (they are few).
-        constexpr int kMine = 512 / kWG;  // candidates per thread
-        uint32_t my[2] = {0, 0};
+        // Exact top-kb among the candidates (every thread takes those of its own wave's list,
+        // one per lane and 64 list slots): a radix select on their keys gives the threshold key
+        // T and the number of entries equal to T to keep; entries above T get consecutive
+        // output slots by a prefix sum over the threads, entries equal to T are ranked among
+        // themselves by index (they are few).
+        constexpr int kMine = kCandPerWave / kWave;  // candidates per thread
+        uint32_t my[kMine], keys[kMine];
         uint32_t have = 0;
 #pragma unroll
         for (int s = 0; s < kMine; ++s) {
-            int i = s * kWG + tid;
-            bool got = false;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                if (!got && i < (int)cnts[w]) {
-                    my[s] = cand[w * kCandPerWave + i];
-                    got = true;
-                }
-                i -= (int)cnts[w];
-                if (i < 0) i = 0x7fffffff;  // already placed, or in a list further on
-            }
+            const uint32_t i = (uint32_t)(s * kWave + lane);
+            const bool got = i < filled;
+            my[s] = got ? mine[i] : 0u;
+            keys[s] = my[s] >> 15;
             have |= (got ? 1u : 0u) << s;
         }
-        const uint32_t keys[2] = {my[0] >> 15, my[1] >> 15};
         if (tid == 0) sh[kShTies] = 0;
         int take_eq, n_eq;
-        const uint32_t T = select_kth_key15<2>(keys, have, kb, hist + kSmallHistWords,
-                                               sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
+        const uint32_t T = select_kth_key15<kMine>(keys, have, kb, hist + kSmallHistWords,
+                                                   sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
         uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the first histograms are free
         constexpr int kMaxTies = 512;
         ok = n_eq <= kMaxTies;
         if (ok) {
             uint32_t n_gt = 0;
 #pragma unroll
-            for (int s = 0; s < 2; ++s) n_gt += (((have >> s) & 1u) != 0 && keys[s] > T) ? 1u : 0u;
+            for (int s = 0; s < kMine; ++s) n_gt += (((have >> s) & 1u) != 0 && keys[s] > T) ? 1u : 0u;
             const uint32_t incl = wg_incl_scan(n_gt, sh, lane, wave);
             uint32_t pos = incl - n_gt;
-            uint32_t tie_idx[2] = {0xffffu, 0xffffu};
+            uint32_t tie_idx[kMine];
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
+            for (int s = 0; s < kMine; ++s) tie_idx[s] = 0xffffu;
+#pragma unroll
+            for (int s = 0; s < kMine; ++s) {
                 if (((have >> s) & 1u) == 0) continue;
                 const uint32_t idx = 32767u - (my[s] & 0x7fffu);
                 if (keys[s] > T) {
@@ -606,7 +601,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
             __syncthreads();
             const int first_eq = kb - take_eq;  // output slots before the ties
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
+            for (int s = 0; s < kMine; ++s) {
                 if (tie_idx[s] == 0xffffu) continue;
                 uint32_t rank = 0;
                 for (int j = 0; j < n_eq; ++j) rank += ties[j] < tie_idx[s] ? 1u : 0u;
