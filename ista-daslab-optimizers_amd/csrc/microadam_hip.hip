@@ -712,6 +712,13 @@ struct FusedBlock {
                     if (!R::kBF16) v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
                     cf[e] = (FULL || off + e < n) ? v : 0.0f;
                 }
+                // bf16 data lies inside its exact statistics and needs no clamp, unless the
+                // step itself is so small that it was rounded coarsely
+                if (R::kBF16 && ex - 32u > 190u) {
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e)
+                        cf[e] = __builtin_amdgcn_fmed3f(cf[e], 0.0f, 15.0f);
+                }
                 float lo = cf[2];
                 lo = __builtin_fmaf(lo, 16.0f, cf[3]);
                 lo = __builtin_fmaf(lo, 16.0f, cf[0]);
@@ -1093,8 +1100,16 @@ struct FusedBlock {
         for (int e = 0; e < kChunk; ++e) {
             float v = div_shared(y[e], dv);
             v = floorf(v + 0.5f);
-            v = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
-            cf[e] = ok ? v : 0.0f;
+            cf[e] = v;
+        }
+        // bf16 data lies inside its exact statistics, so its codes need no clamp unless the
+        // step itself is so small that it was rounded coarsely
+        if (!R::kBF16 || ex - 32u > 190u) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const float v = __builtin_amdgcn_fmed3f(cf[e], 0.0f, 15.0f);
+                cf[e] = ok ? v : 0.0f;
+            }
         }
     }
 

@@ -108,6 +108,16 @@ def test_step_densified_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB,
          expect_route=use_fused)
 
 
+@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
+@pytest.mark.parametrize("scale", [1e-36, 3e-38, 1e-39])
+def test_denormal_scale_gradients(oracle, scale, use_fused):
+    """Gradients so small that quantisation steps and window values are fp32 / bf16 denormals:
+    no flush to zero anywhere, and codes stay inside [0, 15] when the step (max - min) / 15
+    is rounded coarsely."""
+    _run(oracle, [20480 + 4096], torch.bfloat16, 3, 64, 0.01, 0.0, 0.0, 20480, 5, use_fused,
+         grad_scale=scale)
+
+
 def test_config1_plumbing(oracle):
     """The plumbing configuration: one flat fp32 parameter, d = 1,048,576, N(0,1) gradients,
     m=10, k=1 %, q=64, 20 steps, hardware block size."""
