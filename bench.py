@@ -67,6 +67,9 @@ WORKLOADS = {
     "outlier-1.3b": (outlier_1p3b, "bf16", 20, 0.05, 32, 0.0, 1e-3),
     "llama3-8b": (llama3_8b, "bf16", 10, 0.01, 100000, 0.5, 1e-3),
     "plumbing-1m": (lambda: [(1048576,)], "f32", 10, 0.01, 64, 0.0, 1.0),
+    # not a BASELINE configuration: the 7B list with the quantisation block of the reference's
+    # README (quant_block_size=100_000, alpha=0), which takes the two-pass route
+    "llama2-7b-q100k": (llama2_7b, "bf16", 10, 0.01, 100000, 0.0, 1e-3),
 }
 
 
@@ -145,8 +148,8 @@ def cpu_baseline(workload, budget_s=12.0):
 
 def route_label(opt, params):
     """Which route the optimizer takes for the tensors of the list, e.g. "fused" or
-    "densified" when all go one way, else counts per route."""
-    names = {0: "op-by-op", 1: "fused", 2: "densified"}
+    "spanning" when all go one way, else counts per route."""
+    names = {0: "op-by-op", 1: "fused", 2: "spanning"}
     counts = {}
     for p in params:
         r = opt._fusable(p, opt.state[p]) if opt.use_fused else 0

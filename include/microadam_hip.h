@@ -161,32 +161,35 @@ int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
  * return.  Host-only check, launches nothing. */
 int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
 
-/* The whole of update_step (MA:146-328) for alpha > 0 (densify_update_using_ef, MA:296-298 and
- * MA:311-316) when the quantisation blocks are at least as long as the top-k blocks, in two
+/* The whole of update_step (MA:146-328) when the quantisation blocks are at least as long as
+ * the top-k blocks (the reference's documented setting is quant_block_size = 100000), for
+ * alpha == 0 and for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), in two
  * passes per top-k block:
  *   1. a = g + Qinv(e); block top-k -> I[index], V[index]; the residual r is written over g
  *      (the reference's step destroys p.grad as well, MA:190-316) and its min / max per block
  *      to the workspace;
- *   2. min / max of r per quantisation block from the workspace; e1 = Q(r) and Qinv(e1) stay in
- *      registers; window -> Adam direction, + alpha * Qinv(e1); p update (with decoupled weight
- *      decay); error = Q((1 - alpha) * Qinv(e1)), min_vals, max_vals.
+ *   2. min / max of r per quantisation block from the workspace; e1 = Q(r);
+ *      alpha == 0: error = e1, min_vals, max_vals; window -> Adam direction; p update (with
+ *      decoupled weight decay);
+ *      alpha > 0: Qinv(e1) stays in registers; window -> Adam direction, + alpha * Qinv(e1);
+ *      p update; error = Q((1 - alpha) * Qinv(e1)), min_vals, max_vals.
  * The caller advances st['index'] itself.  Conditions (else MA_ERR_NOT_FUSABLE, nothing
- * launched): 0 < alpha < 1 (MA:18); quant_block_size a multiple of 8, not below
+ * launched): 0 <= alpha < 1 (MA:18); quant_block_size a multiple of 8, not below
  * min(d, d_block_size), below 2^30 and covering at most 62 top-k blocks; alignment as for
  * ma_fused_step.
- * workspace: device memory, 16-byte aligned, at least ma_densified_step_workspace() bytes,
+ * workspace: device memory, 16-byte aligned, at least ma_spanning_step_workspace() bytes,
  * owned by the caller; its contents need not survive between calls. */
-int ma_densified_step(const ma_tensor *tensors /* host */, int n_tensors,
+int ma_spanning_step(const ma_tensor *tensors /* host */, int n_tensors,
                       const ma_hyper *hyper /* host */, double alpha, void *workspace,
                       int64_t workspace_bytes, void *stream);
 
-/* Bytes of workspace ma_densified_step needs for this list (16 per top-k block); -1 on bad
+/* Bytes of workspace ma_spanning_step needs for this list (16 per top-k block); -1 on bad
  * arguments.  Host-only. */
-int64_t ma_densified_step_workspace(const ma_tensor *tensors /* host */, int n_tensors,
+int64_t ma_spanning_step_workspace(const ma_tensor *tensors /* host */, int n_tensors,
                                     const ma_hyper *hyper /* host */);
 
-/* 0 if ma_densified_step would accept this tensor, else the MA_ERR_* it would return. */
-int ma_densified_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */,
+/* 0 if ma_spanning_step would accept this tensor, else the MA_ERR_* it would return. */
+int ma_spanning_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */,
                             double alpha);
 
 #ifdef __cplusplus

@@ -957,11 +957,12 @@ struct FusedBlock {
     // =========================================================================================
     // Two-pass route: quantisation blocks of q_span >= block length elements (q_span a
     // multiple of 8), so a top-k block meets at most two of them and their statistics need
-    // every top-k block they cover.  alpha > 0 (MA:296-298, 311-316).
+    // every top-k block they cover.  0 <= alpha < 1 (alpha > 0: MA:296-298, 311-316).
     //   pass 1: a = g + Qinv(e), top-k, window row; the residual r goes to the gradient
     //           buffer, its exact min / max per (block, segment) to the workspace
     //   pass 2: statistics of r from the workspace; e1 = Q(r), d1 = Qinv(e1) in registers;
     //           u = Adam(window) + alpha * d1; p update; r2 = (1 - alpha) * d1; e = Q(r2)
+    //           (alpha == 0: e = e1, u = Adam(window))
     // r2 is a non-decreasing function of the code, and the code of the element, so the
     // statistics of r2 over a quantisation block are r2 at the codes of r's extremes: pass 2
     // needs no second reduction across blocks.
@@ -1050,6 +1051,7 @@ struct FusedBlock {
 
     // Statistics of r (sp_mn / sp_mx) and of r2 (sp2_mn / sp2_mx) for both segments, from the
     // exact extremes of r.
+    template <bool DENSE>
     __device__ __forceinline__ void span_statistics(const BlockGeo &G, const Span &S) {
         float mnx[2], mxx[2];
         gather_extremes(G, S, mnx, mxx);
@@ -1057,6 +1059,11 @@ struct FusedBlock {
         for (int s2 = 0; s2 < 2; ++s2) {
             sp_mn[s2] = f2bf(mnx[s2]);
             sp_mx[s2] = f2bf(mxx[s2]);
+            if (!DENSE) {  // alpha == 0: e = Q(r), the statistics kept are r's
+                sp2_mn[s2] = sp_mn[s2];
+                sp2_mx[s2] = sp_mx[s2];
+                continue;
+            }
             const float mnf = bf2f(sp_mn[s2]);
             const float u = div15(bf2f(sp_mx[s2]) - mnf, d15);
             float x[8], cf[8];
@@ -1229,20 +1236,10 @@ struct FusedBlock {
         for (int c = 0; c < C; ++c) graw[c].load(g, chunk_off<C>(wave, c, lane), n, FULL);
     }
 
-    // d1 = Qinv(Q(r)) of one chunk, (float)code * u + mn as in span_dequant
-    __device__ __forceinline__ void span_requant(int c, float mnf, float u, float (&d1)[8]) {
-        float x[8], cf[8];
-        graw[c].to_float(x);
-        codes8(x, mnf, u, cf);
-#pragma unroll
-        for (int e = 0; e < kChunk; ++e) {
-            float deq = cf[e] * u;
-            d1[e] = deq + mnf;
-        }
-    }
-
-    // p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u; r2 = rne(0 + keep * d1);
-    // e = Q(r2); statistics arrays.  After window_stage.
+    // DENSE (alpha > 0): p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
+    // r2 = rne(0 + keep * d1); e = Q(r2).  Otherwise (alpha == 0): e = Q(r); p += -lr * Adam.
+    // Then the statistics arrays.  After window_stage.
+    template <bool DENSE>
     __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
@@ -1259,8 +1256,17 @@ struct FusedBlock {
             const int off = chunk_off<C>(wave, c, lane);
             if (FULL || off < n) {
                 const bool second = off >= S.bnd;
-                float d1[8];
-                span_requant(c, second ? mn1 : mn0, second ? u1 : u0, d1);
+                float x[8], cf[8], d1[8];
+                graw[c].to_float(x);
+                codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
+                if (DENSE) {
+                    const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        float deq = cf[e] * u;
+                        d1[e] = deq + mnf;
+                    }
+                }
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
                 if (R::kBF16) {
@@ -1279,19 +1285,24 @@ struct FusedBlock {
                     uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
                     uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
                 }
-                float r2[8], cf[8];
+                float r2[8];
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
                     if (apply_decay) pv[e] = to_elem(pv[e] * decay);
-                    const float add = P.alpha * d1[e];
-                    const float ud = to_elem(uv[e] + add);
+                    float ud = uv[e];
+                    if (DENSE) {
+                        const float add = P.alpha * d1[e];
+                        ud = to_elem(uv[e] + add);
+                    }
                     const float prod = neg_lr * ud;
                     pv[e] = pv[e] + prod;
-                    const float keep = P.keep * d1[e];
-                    r2[e] = to_elem(0.0f + keep);
+                    if (DENSE) {
+                        const float keep = P.keep * d1[e];
+                        r2[e] = to_elem(0.0f + keep);
+                    }
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
-                codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
+                if (DENSE) codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
                     if (!FULL && off + e >= n) cf[e] = 0.0f;
@@ -1362,7 +1373,8 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     }
 }
 
-// Two-pass route, see FusedBlock.  PASS 1 / 2; one workgroup per block.
+// Two-pass route, see FusedBlock.  PASS 1; then PASS 2 (alpha > 0) or PASS 3 (alpha == 0); one
+// workgroup per block.
 template <class R, int MIN_WAVES, int PASS>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -1379,9 +1391,9 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             fb.row_in_lds = false;
             fb.load_params_window(G);
             fb.span_load_residual(G);
-            fb.span_statistics(G, S);
+            fb.template span_statistics<PASS == 2>(G, S);
             fb.window_stage(G);
-            fb.span_param_stage(G, S);
+            fb.template span_param_stage<PASS == 2>(G, S);
         }
     };
     if (G.n == R::kC * kRound) {
@@ -1516,10 +1528,14 @@ static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s
         rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
         if (rc) return rc;
         span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
-    } else {
+    } else if (pass == 2) {
         rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
         if (rc) return rc;
         span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
+    } else {
+        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 3>, lds_bytes);
+        if (rc) return rc;
+        span_step_kernel<R, kMinWaves, 3><<<grid, kWG, lds_bytes, s>>>(P);
     }
     return launch_status();
 }
@@ -1584,13 +1600,13 @@ static int fused_check(const ma_tensor *t, const ma_hyper *h) {
 
 constexpr int kSpanMaxBlocks = 64;  // top-k blocks one quantisation block may touch
 
-// the two-pass route: 0 < alpha < 1, quantisation blocks a multiple of 8 and at least as long
+// the two-pass route: 0 <= alpha < 1, quantisation blocks a multiple of 8 and at least as long
 // as the top-k blocks
 static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
     Geometry g;
     const int rc = common_check(t, h, &g);
     if (rc) return rc;
-    if (!(alpha > 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
+    if (!(alpha >= 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
     const int64_t q = h->quant_block_size;
     if (q % 8 != 0 || q < g.dbs || q >= (1LL << 30)) return MA_ERR_NOT_FUSABLE;
     if ((q + g.dbs - 1) / g.dbs + 1 > kSpanMaxBlocks) return MA_ERR_NOT_FUSABLE;
@@ -1847,7 +1863,8 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                          ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
                          : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
             } else {
-                for (int pass = 1; pass <= 2 && rc == 0; ++pass)
+                const int second = alpha > 0.0 ? 2 : 3;
+                for (int pass = 1; pass <= second && rc == 0; pass += second - 1)
                     rc = h->dtype == MA_BF16
                              ? launch_span<RegsBF16>(C, pass, (unsigned)items, P.L.total, s, P)
                              : launch_span<RegsF32>(C, pass, (unsigned)items, P.L.total, s, P);
@@ -1903,11 +1920,11 @@ int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, vo
     return step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0);
 }
 
-int ma_densified_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {
+int ma_spanning_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {
     return span_check(tensor, hyper, alpha);
 }
 
-int64_t ma_densified_step_workspace(const ma_tensor *tensors, int n_tensors, const ma_hyper *h) {
+int64_t ma_spanning_step_workspace(const ma_tensor *tensors, int n_tensors, const ma_hyper *h) {
     if (!tensors || !h || n_tensors < 0) return -1;
     int64_t need = 0;
     for (int i = 0; i < n_tensors; ++i) {
@@ -1917,7 +1934,7 @@ int64_t ma_densified_step_workspace(const ma_tensor *tensors, int n_tensors, con
     return need;
 }
 
-int ma_densified_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, double alpha,
+int ma_spanning_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, double alpha,
                       void *workspace, int64_t workspace_bytes, void *stream) {
     return step_impl(tensors, n_tensors, h, stream, true, alpha, workspace, workspace_bytes);
 }

@@ -81,7 +81,7 @@ class MicroAdam(torch.optim.Optimizer):
         self.use_fused = True
         self._fused_cache = None
         self._route = {}
-        self._workspace = None  # device scratch of the densified route, grown on demand
+        self._workspace = None  # device scratch of the spanning route, grown on demand
 
     # ------------------------------------------------------------------ state (micro_adam.py:61-94)
     def _initialize_parameter_state(self, p, lr, wd):
@@ -143,7 +143,7 @@ class MicroAdam(torch.optim.Optimizer):
         norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe = 0, 0, 0, 0, 0, 0
         logging_step = self._logging_active() and self.steps % self.log_interval == 0
 
-        fused, densified = [], []  # (p, st, lr, wd)
+        fused, spanning = [], []  # (p, st, lr, wd)
         for group in self.param_groups:
             lr = group['lr']
             wd = group.get('weight_decay', self.weight_decay)
@@ -163,7 +163,7 @@ class MicroAdam(torch.optim.Optimizer):
 
                 route = self._fusable(p, st) if self.use_fused and not logging_step else 0
                 if route:
-                    (fused if route == 1 else densified).append((p, st, lr, wd))
+                    (fused if route == 1 else spanning).append((p, st, lr, wd))
                     continue
 
                 nqe, ng, nu, ne, sp_u, sp_qe = self.update_step(p, lr, wd, logging_step)
@@ -176,8 +176,8 @@ class MicroAdam(torch.optim.Optimizer):
 
         if fused:
             self._fused_step(fused)
-        if densified:
-            self._fused_step(densified, densified=True)
+        if spanning:
+            self._fused_step(spanning, spanning=True)
 
         time_end = time.time()
         elapsed_step = time_end - time_start
@@ -236,9 +236,9 @@ class MicroAdam(torch.optim.Optimizer):
 
     def _fusable(self, p, st):
         """0: op-by-op route; 1: ma_fused_step (alpha == 0, quantisation blocks inside the top-k
-        blocks); 2: ma_densified_step (alpha > 0, quantisation blocks at least as long as the
+        blocks); 2: ma_spanning_step (0 <= alpha < 1, quantisation blocks at least as long as the
         top-k blocks).  The conditions are those of include/microadam_hip.h."""
-        if self.alpha < 0:
+        if not 0 <= self.alpha < 1:
             return 0
         g = p.grad
         if g.dtype != p.dtype or not p.is_contiguous() or not g.is_contiguous():
@@ -251,20 +251,19 @@ class MicroAdam(torch.optim.Optimizer):
             common = (self.m <= _hip.MA_MAX_WINDOW and dbs <= 32768
                       and (d <= self.d_block_size or dbs % 8 == 0))
             route = 0
-            if common and self.alpha == 0:
-                if (8 <= q <= 512 and (q & (q - 1)) == 0 and d >= q
-                        and (d <= self.d_block_size or dbs % q == 0)):
-                    route = 1
-            elif common and 0 < self.alpha < 1:
-                if q % 8 == 0 and dbs <= q < (1 << 30) and (q + dbs - 1) // dbs + 1 <= 64:
-                    route = 2
+            if (common and self.alpha == 0 and 8 <= q <= 512 and (q & (q - 1)) == 0 and d >= q
+                    and (d <= self.d_block_size or dbs % q == 0)):
+                route = 1
+            elif (common and q % 8 == 0 and dbs <= q < (1 << 30)
+                  and (q + dbs - 1) // dbs + 1 <= 64):
+                route = 2
             self._route[id(p)] = route
         return route
 
-    def _fused_step(self, items, densified=False):
+    def _fused_step(self, items, spanning=False):
         n = len(items)
-        key = (densified,) + tuple(id(p) for p, _, _, _ in items)
-        cache = self._fused_cache.get(densified) if self._fused_cache else None
+        key = (spanning,) + tuple(id(p) for p, _, _, _ in items)
+        cache = self._fused_cache.get(spanning) if self._fused_cache else None
         if cache is None or cache[0] != key:
             arr = (_hip.MaTensor * n)()
             for t, (p, st, _, _) in zip(arr, items):
@@ -273,7 +272,7 @@ class MicroAdam(torch.optim.Optimizer):
             cache = (key, arr)
             if self._fused_cache is None:
                 self._fused_cache = {}
-            self._fused_cache[densified] = cache
+            self._fused_cache[spanning] = cache
         arr = cache[1]
         for t, (p, st, lr, wd) in zip(arr, items):
             t.p = p.data_ptr()
@@ -298,18 +297,18 @@ class MicroAdam(torch.optim.Optimizer):
             h = _hip.MaHyper(self.steps, self.m, _hip.MA_BF16 if dtype == torch.bfloat16 else _hip.MA_F32,
                              self.quant_block_size, self.d_block_size, self.k_init, self.beta1,
                              self.beta2, self.eps)
-            if not densified:
+            if not spanning:
                 rc = _hip.lib.ma_fused_step(sub, cnt, ctypes.byref(h), _hip.stream_ptr())
                 _hip.check(rc, "ma_fused_step")
                 continue
-            need = _hip.lib.ma_densified_step_workspace(sub, cnt, ctypes.byref(h))
+            need = _hip.lib.ma_spanning_step_workspace(sub, cnt, ctypes.byref(h))
             ws = self._workspace
             if ws is None or ws.numel() < need or ws.device != items[idxs[0]][0].device:
                 ws = self._workspace = torch.empty(max(need, 16), dtype=torch.uint8,
                                                    device=items[idxs[0]][0].device)
-            rc = _hip.lib.ma_densified_step(sub, cnt, ctypes.byref(h), float(self.alpha),
+            rc = _hip.lib.ma_spanning_step(sub, cnt, ctypes.byref(h), float(self.alpha),
                                             ws.data_ptr(), ws.numel(), _hip.stream_ptr())
-            _hip.check(rc, "ma_densified_step")
+            _hip.check(rc, "ma_spanning_step")
         for _, st, _, _ in items:
             st['index'] = (st['index'] + 1) % self.m
 

@@ -75,17 +75,18 @@ def test_fused_step_check_rejects_bad_layouts():
     assert chk() == -3
 
 
-def test_densified_step_check_and_workspace():
-    """Host-only validation of ma_densified_step's conditions and its workspace size."""
+def test_spanning_step_check_and_workspace():
+    """Host-only validation of ma_spanning_step's conditions and its workspace size."""
     from ista_daslab_optimizers import _hip
     t = _hip.MaTensor()
     for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
         setattr(t, f, 0x10000)
     t.d, t.k, t.lr, t.weight_decay, t.index = 20480 * 2 + 4096, 205 * 2 + 41, 1e-3, 0.0, 0
     h = _hip.MaHyper(1, 10, _hip.MA_BF16, 100000, 20480, 0.01, 0.9, 0.999, 1e-8)
-    chk = lambda a: _hip.lib.ma_densified_step_check(ctypes.byref(t), ctypes.byref(h), a)
+    chk = lambda a: _hip.lib.ma_spanning_step_check(ctypes.byref(t), ctypes.byref(h), a)
     assert chk(0.5) == 0
-    assert chk(0.0) == _hip.MA_ERR_NOT_FUSABLE      # alpha == 0 is ma_fused_step's case
+    assert chk(0.0) == 0
+    assert chk(-2.0) == _hip.MA_ERR_NOT_FUSABLE
     assert chk(1.0) == _hip.MA_ERR_NOT_FUSABLE      # micro_adam.py:18 asks for alpha < 1
     h.quant_block_size = 100001                     # not a multiple of 8
     assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
@@ -95,7 +96,7 @@ def test_densified_step_check_and_workspace():
     assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
     h.quant_block_size = 100000
     arr = (_hip.MaTensor * 2)(t, t)
-    assert _hip.lib.ma_densified_step_workspace(arr, 2, ctypes.byref(h)) == 2 * 3 * 16
+    assert _hip.lib.ma_spanning_step_workspace(arr, 2, ctypes.byref(h)) == 2 * 3 * 16
     # too small a workspace is refused before anything is launched
-    rc = _hip.lib.ma_densified_step(arr, 2, ctypes.byref(h), 0.5, 0x10000, 16, None)
+    rc = _hip.lib.ma_spanning_step(arr, 2, ctypes.byref(h), 0.5, 0x10000, 16, None)
     assert rc == -1  # MA_ERR_ARG

@@ -119,7 +119,7 @@ def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, step
             assert not bool((moved & ~touched).any())
 
 
-def test_densified_and_opbyop_agree_at_llama3_shapes():
+def test_spanning_and_opbyop_agree_at_llama3_shapes():
     """alpha = 0.5 with quantisation blocks of 100000 elements (they straddle the 20480-element
     top-k blocks): the two-pass fused route and the op-by-op kernels, which form the statistics
     in different ways, end in bit-identical parameters and state."""

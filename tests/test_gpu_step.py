@@ -79,7 +79,7 @@ GENERAL_CASES = [
     ([4100, 33], torch.bfloat16, 3, 1000, 0.01, 0.5, 0.0, 1024, 7),
     ([999], torch.float32, 2, 100, 0.03, 0.25, 0.01, 400, 5),
     ([20480 * 3 + 77], torch.bfloat16, 4, 100001, 0.01, 0.5, 0.0, 20480, 6),
-    ([50, 20], torch.bfloat16, 3, 64, 0.1, 0.0, 0.0, 20480, 4),
+    ([50, 20], torch.bfloat16, 3, 60, 0.1, 0.0, 0.0, 20480, 4),
     # alpha == -2: the quantisation error goes straight into the parameters (micro_adam.py:238-273)
     ([20480 + 4096, 300], torch.bfloat16, 4, 64, 0.01, -2, 0.0, 20480, 6),
     ([3000], torch.float32, 3, 64, 0.02, -2, 0.05, 1024, 5),
@@ -91,19 +91,23 @@ def test_step_general_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, s
     _run(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, True, expect_route=False)
 
 
-DENSIFIED_CASES = [
-    # alpha > 0 with quantisation blocks at least as long as the top-k blocks: three-pass route
+SPANNING_CASES = [
+    # quantisation blocks at least as long as the top-k blocks: two-pass route
     ([20480 * 5 + 77], torch.bfloat16, 10, 100000, 0.01, 0.5, 0.0, 20480, 12),
     ([20480 * 12 + 4096, 4096, 1000], torch.bfloat16, 4, 24576, 0.01, 0.3, 0.01, 20480, 8),
     ([5000, 3000], torch.float32, 3, 2048, 0.02, 0.25, 0.0, 1024, 6),
     ([40000], torch.bfloat16, 3, 20480, 0.01, 0.9, 0.0, 20480, 5),
     ([512 * 9 + 100], torch.bfloat16, 3, 520, 0.02, 0.5, 0.0, 512, 6),
+    # alpha == 0 with long quantisation blocks (the reference's documented quant_block_size)
+    ([20480 * 5 + 77, 4096], torch.bfloat16, 10, 100000, 0.01, 0.0, 0.0, 20480, 12),
+    ([5000, 3000], torch.float32, 3, 2048, 0.02, 0.0, 0.01, 1024, 6),
+    ([50, 20], torch.bfloat16, 3, 64, 0.1, 0.0, 0.0, 20480, 4),       # d < q
 ]
 
 
-@pytest.mark.parametrize("use_fused", [True, False], ids=["densified", "opbyop"])
-@pytest.mark.parametrize("sizes,dtype,m,q,k_init,alpha,wd,DB,steps", DENSIFIED_CASES)
-def test_step_densified_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused):
+@pytest.mark.parametrize("use_fused", [True, False], ids=["spanning", "opbyop"])
+@pytest.mark.parametrize("sizes,dtype,m,q,k_init,alpha,wd,DB,steps", SPANNING_CASES)
+def test_step_spanning_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused):
     _run(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused, zero_step=2,
          expect_route=use_fused)
 
