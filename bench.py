@@ -170,6 +170,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB -> 1 GiB device copy, as the known-size kernel "
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled against")
+    ap.add_argument("--storage", choices=["bf16", "f32"], default=None,
+                    help="override the element type of parameters and gradients")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -180,6 +182,8 @@ def main():
     shapes_fn, dtype, m, k_init, q, alpha, gstd = WORKLOADS[args.workload]
     if args.warmup is None:
         args.warmup = m + 2
+    if args.storage is not None:
+        dtype = args.storage
     shapes = shapes_fn()
     tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
     dev = torch.device("cuda:0")
@@ -255,7 +259,8 @@ def main():
                    "route": route_label(opt, params)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op)),
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op))
+                     if args.storage is None else None,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},
     }
