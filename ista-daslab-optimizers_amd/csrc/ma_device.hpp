@@ -182,7 +182,6 @@ struct RegsBF16 {
     static constexpr bool kBF16 = true;
     static constexpr int kElemBytes = 2;
     typedef uint16_t elem_t;
-    typedef uint16_t slot_t;  // LDS cell per coordinate: window bookkeeping, later the update's bits
     uint32_t w[C][4];         // two bf16 per register
 
     __device__ __forceinline__ uint32_t key(int c, int e) const {
@@ -212,7 +211,6 @@ struct RegsF32 {
     static constexpr bool kBF16 = false;
     static constexpr int kElemBytes = 4;
     typedef float elem_t;
-    typedef uint32_t slot_t;
     float w[C][8];
 
     __device__ __forceinline__ uint32_t key(int c, int e) const {

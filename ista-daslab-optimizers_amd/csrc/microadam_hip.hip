@@ -228,12 +228,13 @@ __global__ __launch_bounds__(kWG) void param_update_kernel(int64_t d, T *p, cons
 struct LdsMap {
     int off_sel_idx;  // uint16[kb_max]
     int off_sel_val;  // uint16[kb_max]
-    int off_slot;     // slot_t[slot_cells]
+    int off_slot;     // slot_cells cells of cell_bytes
     int off_union;    // histograms and candidate lists during selection, then the window stage's arrays
     int slot_cells;   // multiple of 8, >= longest block
     int z_cap;        // entries the window stage's arrays hold
     int sub_len;      // coordinates handled per window pass
     int fast_cap;     // entries the one-pass window stage has room for, 0: none
+    int cell_bytes;   // width of a slot cell: 2, or 4 for fp32 data in the general window stage
     int total;        // bytes
 };
 constexpr int kMiscBytes = 256;  // the kSh* words at the very start
@@ -439,13 +440,17 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
 template <class R, bool FULL, int QL>
 struct FusedBlock {
     typedef typename R::elem_t elem_t;
-    typedef typename R::slot_t slot_t;
     static constexpr int C = R::kC;
 
     const FusedParams &P;
     uint32_t *sh, *counter, *hist;
     uint16_t *sel_idx, *sel_val, *coord;
-    slot_t *slot;
+    // One LDS cell per coordinate of the block.  16 bits wide for bf16 data (window bookkeeping,
+    // then the update's bf16 bits) and in the one-pass window stage for fp32 data (bookkeeping,
+    // then 1 + the record that holds the update); 32 bits (the update's bits) for fp32 data in
+    // the general window stage.
+    uint16_t *cell16;
+    uint32_t *cell32;
     float *z1, *z2;
     int tid, lane, wave, q_shift, ql;
     bool slot_clear;  // the slot cells are already zero when the update stage begins
@@ -472,7 +477,8 @@ struct FusedBlock {
         counter = sh + kShCounter;
         sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
         sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
-        slot = reinterpret_cast<slot_t *>(lds + P.L.off_slot);
+        cell16 = reinterpret_cast<uint16_t *>(lds + P.L.off_slot);
+        cell32 = reinterpret_cast<uint32_t *>(lds + P.L.off_slot);
         hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
         z1 = reinterpret_cast<float *>(lds + P.L.off_union);
         z2 = z1 + P.L.z_cap;
@@ -619,7 +625,7 @@ struct FusedBlock {
 #else
         if constexpr (FULL && R::kBF16) {
             if (kb <= kWG) {
-                topk_done = fast_topk_bf16(r, kb, reinterpret_cast<uint16_t *>(slot), hist, sh,
+                topk_done = fast_topk_bf16(r, kb, cell16, hist, sh,
                                            sel_idx, sel_val, pt);
                 launder(r);
                 pt.mark(7);
@@ -759,8 +765,8 @@ struct FusedBlock {
         const TensorDesc &D = G.D;
         if (!slot_clear) {
             __syncthreads();  // the LDS of the selection is reused below
-            for (int i = tid; i < P.L.slot_cells * (int)sizeof(slot_t) / 16; i += kWG)
-                reinterpret_cast<uint4 *>(slot)[i] = make_uint4(0, 0, 0, 0);
+            for (int i = tid; i < P.L.slot_cells * P.L.cell_bytes / 16; i += kWG)
+                reinterpret_cast<uint4 *>(cell16)[i] = make_uint4(0, 0, 0, 0);
         }
 #if defined(MA_ABLATE) && MA_ABLATE == 3
         if (false) {
@@ -773,7 +779,7 @@ struct FusedBlock {
             // others go to a list; the entry of the lowest row owns the coordinate, hands out
             // one link cell per later row, the later rows file their list position there by
             // rank, and the owner adds them up in that order, which is the order of the rows.
-            uint32_t *mcount = sh + kShCounter, *lcount = sh + kShLinks;
+            uint32_t *mcount = sh + kShCounter, *lcount = sh + kShLinks, *scount = sh + kShTies;
             float *f1 = z1, *f2 = z2;
             const int cap = P.L.z_cap;
             uint16_t *mI = coord, *mR = mI + cap, *mM = mR + cap, *link = mM + cap;
@@ -781,7 +787,7 @@ struct FusedBlock {
                 sh[kShW1 + tid] = __float_as_uint(P.W.w1[tid]);
                 sh[kShW2 + tid] = __float_as_uint(P.W.w2[tid]);
             }
-            if (tid == 0) *mcount = *lcount = 0;
+            if (tid == 0) *mcount = *lcount = *scount = 0;
             const int wave_first = __builtin_amdgcn_readfirstlane(wave) * kWave;
             const int entries = rows * kb;
             const float rkb = __builtin_amdgcn_rcpf((float)kb);
@@ -804,11 +810,7 @@ struct FusedBlock {
                         // are all (index 0, value 0)); idx < n keeps a corrupt index inside
                         if (idx < (uint32_t)n && (vb & 0x7fffu) != 0) {
                             tag = idx | (uint32_t)row << 16;
-                            if (sizeof(slot_t) == 2)
-                                atomicOr(reinterpret_cast<uint32_t *>(slot) + (idx >> 1),
-                                         (1u << row) << ((idx & 1u) * 16));
-                            else
-                                atomicOr(reinterpret_cast<uint32_t *>(slot) + idx, 1u << row);
+                            atomicOr(cell32 + (idx >> 1), (1u << row) << ((idx & 1u) * 16));
                         }
                     }
                 }
@@ -820,7 +822,7 @@ struct FusedBlock {
                 const uint32_t tag = entI[i];
                 if (tag != 0xffffffffu) {
                     const uint32_t idx = tag & 0xffffu, row = tag >> 16;
-                    const uint32_t mask = slot[idx];
+                    const uint32_t mask = cell16[idx];
                     const float v = bf2f(entV[i]);
                     const float a1 = __uint_as_float(sh[kShW1 + row]) * v;
                     const float vv = v * v;
@@ -828,7 +830,14 @@ struct FusedBlock {
                     if (mask == 1u << row) {
                         const float u =
                             adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
-                        slot[idx] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                        if (R::kBF16) {
+                            cell16[idx] = (uint16_t)f2bf(u);
+                        } else {  // fp32: the update keeps its bits in a record of its own,
+                                  // handed out from the top of the list arrays
+                            const uint32_t s = (uint32_t)cap - 1u - atomicAdd(scount, 1u);
+                            f1[s] = u;
+                            cell16[idx] = (uint16_t)(s + 1u);
+                        }
                     } else {
                         const uint32_t s = atomicAdd(mcount, 1u);
                         f1[s] = a1;
@@ -845,13 +854,13 @@ struct FusedBlock {
             for (int s = tid; s < listed; s += kWG) {
                 const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
                 if (below == 0)
-                    slot[mI[s]] = (slot_t)atomicAdd(lcount, (uint32_t)__popc(mask) - 1u);
+                    cell16[mI[s]] = (uint16_t)atomicAdd(lcount, (uint32_t)__popc(mask) - 1u);
             }
             __syncthreads();
             for (int s = tid; s < listed; s += kWG) {
                 const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
                 if (below != 0) {
-                    const uint32_t at = (uint32_t)slot[mI[s]] + (uint32_t)__popc(below) - 1u;
+                    const uint32_t at = (uint32_t)cell16[mI[s]] + (uint32_t)__popc(below) - 1u;
                     if (at < (uint32_t)cap) link[at] = (uint16_t)s;
                 }
             }
@@ -859,7 +868,7 @@ struct FusedBlock {
             for (int s = tid; s < listed; s += kWG) {
                 const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
                 if (below == 0) {
-                    const uint32_t idx = mI[s], base = slot[idx];
+                    const uint32_t idx = mI[s], base = cell16[idx];
                     float s1 = 0.0f + f1[s], s2 = 0.0f + f2[s];
                     const int later = __popc(mask) - 1;
                     for (int r = 0; r < later; ++r) {
@@ -872,7 +881,12 @@ struct FusedBlock {
                         s2 = s2 + f2[o];
                     }
                     const float u = adam_direction(s1, s2, P.W.s1, P.W.s2, P.W.eps);
-                    slot[idx] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                    if (R::kBF16) {
+                        cell16[idx] = (uint16_t)f2bf(u);
+                    } else {  // the owner's record has given its sums and takes the update
+                        f1[s] = u;
+                        cell16[idx] = (uint16_t)(s + 1);
+                    }
                 }
             }
             __syncthreads();
@@ -898,13 +912,44 @@ struct FusedBlock {
                 for (int c = tid; c < hi - lo; c += kWG) {
                     if (z1[c] != 0.0f || z2[c] != 0.0f) {
                         const float u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
-                        slot[lo + c] = R::kBF16 ? (slot_t)f2bf(u) : (slot_t)__float_as_uint(u);
+                        if (R::kBF16) cell16[lo + c] = (uint16_t)f2bf(u);
+                        else cell32[lo + c] = __float_as_uint(u);
                     }
                 }
                 __syncthreads();
             }
         }
         pt.mark(15);
+    }
+
+    // the Adam direction of the 8 coordinates at `off`, as the window stage left it in the cells
+    __device__ __forceinline__ void update8(int off, float (&uv)[8]) const {
+        if (R::kBF16 || P.L.cell_bytes == 2) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(cell16 + off);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            if (R::kBF16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uv[2 * i] = __uint_as_float(w[i] << 16);
+                    uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                }
+            } else {
+                const float *rec = z1;  // record s holds the update of the coordinate with cell s + 1
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t c = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+                    uv[i] = 0.0f;
+                    if (c != 0) uv[i] = rec[c - 1];
+                }
+            }
+        } else {
+            const uint4 a = *reinterpret_cast<const uint4 *>(cell32 + off);
+            const uint4 b2 = *reinterpret_cast<const uint4 *>(cell32 + off + 4);
+            uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
+            uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
+            uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
+            uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
+        }
     }
 
     __device__ __forceinline__ void param_stage(const BlockGeo &G) {
@@ -919,22 +964,7 @@ struct FusedBlock {
             if (FULL || off < n) {
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
-                if (R::kBF16) {
-                    const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
-                    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        uv[2 * i] = __uint_as_float(w[i] << 16);
-                        uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                    }
-                } else {
-                    const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
-                    const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
-                    uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
-                    uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
-                    uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
-                    uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
-                }
+                update8(off, uv);
                 if (apply_decay) {
 #pragma unroll
                     for (int e = 0; e < kChunk; ++e) {
@@ -1269,22 +1299,7 @@ struct FusedBlock {
                 }
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
-                if (R::kBF16) {
-                    const uint4 q = *reinterpret_cast<const uint4 *>(slot + off);
-                    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        uv[2 * i] = __uint_as_float(w[i] << 16);
-                        uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                    }
-                } else {
-                    const uint4 a = *reinterpret_cast<const uint4 *>(slot + off);
-                    const uint4 b2 = *reinterpret_cast<const uint4 *>(slot + off + 4);
-                    uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
-                    uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
-                    uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
-                    uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
-                }
+                update8(off, uv);
                 float r2[8];
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
@@ -1412,19 +1427,21 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
 static inline int align16(int x) { return (x + 15) & ~15; }
 
 // LDS plan for a block kernel: longest block `dbs_max`, most entries per block row `kb_max`,
-// window length m, bytes per slot cell.
-static LdsMap plan_lds(int dbs_max, int kb_max, int m, int slot_bytes, bool one_pass = true) {
+// window length m, bytes per element of the data.
+static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_pass = true) {
     LdsMap L;
     L.off_sel_idx = kMiscBytes;
     L.off_sel_val = L.off_sel_idx + align16(kb_max * 2);
     L.off_slot = L.off_sel_val + align16(kb_max * 2);
     L.slot_cells = (dbs_max + 7) & ~7;
-    L.off_union = L.off_slot + align16(L.slot_cells * slot_bytes);
     // one-pass window stage: two floats and four 16-bit words per entry; otherwise the block is
     // walked in coordinate ranges of at most 4096 with two dense fp32 arrays
     const int64_t entries = (int64_t)m * kb_max;
+    const bool fast = one_pass && entries <= kEnt * kWG && m <= kFastRows;
+    L.cell_bytes = (elem_bytes == 2 || fast) ? 2 : 4;
+    L.off_union = L.off_slot + align16(L.slot_cells * L.cell_bytes);
     L.fast_cap = 0;
-    if (one_pass && entries <= kEnt * kWG && m <= kFastRows) {
+    if (fast) {
         L.fast_cap = L.z_cap = (int)(entries < 8 ? 8 : entries);
         L.sub_len = L.slot_cells;
     } else {
@@ -1831,7 +1848,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     while (!span && (1LL << q_shift) < h->quant_block_size) ++q_shift;
     WindowWeights W;
     window_weights(h->t, h->m, h->beta1, h->beta2, h->eps, &W);
-    const int slot_bytes = h->dtype == MA_BF16 ? 2 : 4;
+    const int elem_bytes = h->dtype == MA_BF16 ? 2 : 4;
 
     // Work is handed out in launches of at most kTensorsPerLaunch tensors (their descriptors
     // travel by value), one workgroup per top-k block, grouped by register-tile class so that
@@ -1849,7 +1866,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             if (count == 0) return 0;
             P.n_tensors = count;
             P.W = W;
-            P.L = plan_lds(dbs_max, kb_max, h->m, slot_bytes);
+            P.L = plan_lds(dbs_max, kb_max, h->m, elem_bytes);
             P.d_block_size = d_block_size;
             P.q_shift = q_shift;
             P.total_items = (int32_t)items;
