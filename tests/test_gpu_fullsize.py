@@ -37,17 +37,18 @@ def _grads(shape, kind, step, dtype):
 
 
 CASES = [
-    # shapes, m, k_init, q, grad kind, steps
-    ([(32000, 4096), (11008, 4096), (4096, 4096), (4096,)], 10, 0.01, 64, "normal", 12),
-    ([(50304, 2048), (2048, 8192)], 20, 0.05, 32, "outlier", 4),
+    # shapes, m, k_init, q, grad kind, steps, dtype
+    ([(32000, 4096), (11008, 4096), (4096, 4096), (4096,)], 10, 0.01, 64, "normal", 12,
+     torch.bfloat16),
+    ([(50304, 2048), (2048, 8192)], 20, 0.05, 32, "outlier", 4, torch.bfloat16),
+    ([(11008, 4096), (4096,)], 10, 0.01, 64, "normal", 12, torch.float32),
 ]
 
 
-@pytest.mark.parametrize("shapes,m,k_init,q,kind,steps", CASES)
-def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, steps):
+@pytest.mark.parametrize("shapes,m,k_init,q,kind,steps,dtype", CASES)
+def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, steps, dtype):
     from ista_daslab_optimizers import MicroAdam
     import ista_daslab_cuda_micro_adam as ext
-    dtype = torch.bfloat16
     torch.manual_seed(0)
     pa = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in shapes]
     pb = [torch.nn.Parameter(p.detach().clone()) for p in pa]
@@ -89,7 +90,7 @@ def test_fused_and_opbyop_agree_and_select_topk(shapes, m, k_init, q, kind, step
             assert int(pos.max()) < a.numel()
             assert torch.unique(pos).numel() == k, "duplicate index in a block row"
             mag = a.float().abs()
-            assert torch.equal(sa["V"][row], a[pos]), "window values are not a[I]"
+            assert torch.equal(sa["V"][row], a[pos].to(torch.bfloat16)), "window values are not a[I]"
             sel = torch.zeros_like(mag, dtype=torch.bool)
             sel[pos] = True
             nblk = (a.numel() + dbs - 1) // dbs
