@@ -70,6 +70,8 @@ WORKLOADS = {
     # not a BASELINE configuration: the 7B list with the quantisation block of the reference's
     # README (quant_block_size=100_000, alpha=0), which takes the two-pass route
     "llama2-7b-q100k": (llama2_7b, "bf16", 10, 0.01, 100000, 0.0, 1e-3),
+    # not a BASELINE configuration either: the 7B list with alpha > 0 and short quantisation blocks
+    "llama2-7b-alpha": (llama2_7b, "bf16", 10, 0.01, 64, 0.5, 1e-3),
 }
 
 
@@ -149,7 +151,7 @@ def cpu_baseline(workload, budget_s=12.0):
 def route_label(opt, params):
     """Which route the optimizer takes for the tensors of the list, e.g. "fused" or
     "spanning" when all go one way, else counts per route."""
-    names = {0: "op-by-op", 1: "fused", 2: "spanning"}
+    names = {0: "op-by-op", 1: "fused", 2: "spanning", 3: "fused-densified"}
     counts = {}
     for p in params:
         r = opt._fusable(p, opt.state[p]) if opt.use_fused else 0

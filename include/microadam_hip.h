@@ -161,6 +161,13 @@ int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
  * return.  Host-only check, launches nothing. */
 int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
 
+/* ma_fused_step for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), same
+ * conditions, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and
+ * statistics; window -> Adam direction, + alpha * Qinv(e1); p update; the error feedback that is
+ * stored is Q((1 - alpha) * Qinv(e1)) with statistics of its own. */
+int ma_fused_step_densified(const ma_tensor *tensors /* host */, int n_tensors,
+                            const ma_hyper *hyper /* host */, double alpha, void *stream);
+
 /* The whole of update_step (MA:146-328) when the quantisation blocks are at least as long as
  * the top-k blocks (the reference's documented setting is quant_block_size = 100000), for
  * alpha == 0 and for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), in two

@@ -984,6 +984,119 @@ struct FusedBlock {
         pt.mark(16);
     }
 
+    // ---- alpha > 0 with quantisation blocks inside the block (MA:296-298, 311-316) -------------
+    // quantize_dense replaces quantize: e1 = Q(r) is kept as packed codes with its statistics
+    // (for the update, which adds alpha * Qinv(e1)), and the error feedback that is stored is
+    // Q of r2 = (1 - alpha) * Qinv(e1) with statistics of its own.
+    uint32_t dcodes[C], dstat[C];  // e1 of the chunk; its min | max << 16 (bf16 bits)
+
+    __device__ __forceinline__ void quantize_dense(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        uint8_t *err = G.D.err + (G.e0 >> 1);
+        uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float x[8];
+            float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                x[e] = r.val(c, e);
+                if (FULL || off + e < n) {
+                    mn = fmin_raw(mn, x[e]);
+                    mx = fmax_raw(mx, x[e]);
+                }
+            }
+            group_minmax<QL>(mn, mx, ql);
+            const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
+            dstat[c] = mnb | mxb << 16;
+            dcodes[c] = 0;
+            float r2[8];
+            float mn2 = INFINITY, mx2 = -INFINITY;
+            if (FULL || off < n) {
+                const float mnf = bf2f(mnb);
+                const float u = div15(bf2f(mxb) - mnf, d15);
+                float cf[8];
+                codes8(x, mnf, u, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                dcodes[c] = pack_codes(cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    float deq = cf[e] * u;
+                    deq = deq + mnf;
+                    const float keep = P.keep * deq;
+                    r2[e] = to_elem(0.0f + keep);
+                    if (FULL || off + e < n) {
+                        mn2 = fmin_raw(mn2, r2[e]);
+                        mx2 = fmax_raw(mx2, r2[e]);
+                    }
+                }
+            }
+            group_minmax<QL>(mn2, mx2, ql);
+            const uint32_t mn2b = f2bf(mn2), mx2b = f2bf(mx2);
+            if (FULL || off < n) {
+                if ((lane & (ql - 1)) == 0) {
+                    const unsigned qb = (unsigned)off >> q_shift;
+                    mnp[qb] = (uint16_t)mn2b;
+                    mxp[qb] = (uint16_t)mx2b;
+                }
+                const float m2f = bf2f(mn2b);
+                const float u2 = div15(bf2f(mx2b) - m2f, d15);
+                float cf[8];
+                codes8(r2, m2f, u2, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        pt.mark(11);
+    }
+
+    // p = p * decay; u = rne(Adam + alpha * Qinv(e1)); p += -lr * u.  After window_stage.
+    __device__ __forceinline__ void param_stage_dense(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                update8(off, uv);
+                const float mnf = bf2f(dstat[c] & 0xffffu);
+                const float u = div15(bf2f(dstat[c] >> 16) - mnf, d15);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                    const uint32_t code = (dcodes[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                    float deq = (float)code * u;
+                    deq = deq + mnf;
+                    const float add = P.alpha * deq;
+                    const float ud = to_elem(uv[e] + add);
+                    const float prod = neg_lr * ud;
+                    pv[e] = pv[e] + prod;
+                }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
     // =========================================================================================
     // Two-pass route: quantisation blocks of q_span >= block length elements (q_span a
     // multiple of 8), so a top-k block meets at most two of them and their statistics need
@@ -1356,35 +1469,39 @@ __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
 
 // One workgroup per block: any block shape.  Tensor i contributes its blocks
 // blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
-template <class R, int MIN_WAVES, int QL>
+template <class R, int MIN_WAVES, int QL, bool DENSE = false>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int ti = find_tensor(P, (int)blockIdx.x);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
+    auto run = [&](auto &fb) {
+        fb.load_params_window(G);
+        fb.load_grad_inputs(G);
+        fb.dequant(G);
+        fb.topk_and_row(G);
+        if constexpr (DENSE) {
+            fb.quantize_dense(G);
+            fb.window_stage(G);
+            fb.param_stage_dense(G);
+        } else {
+            fb.quantize(G);
+            fb.update(G);
+        }
+    };
 #ifdef MA_ANALYZE_FULL_ONLY  // development aid: a listing with the full-block path alone
     if (true) {
 #else
     if (G.n == R::kC * kRound) {
 #endif
         FusedBlock<R, true, QL> fb(P, lds);
-        fb.load_params_window(G);
-        fb.load_grad_inputs(G);
-        fb.dequant(G);
-        fb.topk_and_row(G);
-        fb.quantize(G);
-        fb.update(G);
+        run(fb);
 #ifdef MA_ANALYZE_FULL_ONLY
     } else if (false) {
 #else
     } else {
 #endif
         FusedBlock<R, false, QL> fb(P, lds);
-        fb.load_params_window(G);
-        fb.load_grad_inputs(G);
-        fb.dequant(G);
-        fb.topk_and_row(G);
-        fb.quantize(G);
-        fb.update(G);
+        run(fb);
     }
 }
 
@@ -1515,12 +1632,25 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
     return MA_ERR_BLOCK_SIZE;
 }
 
-template <class R, int QL>
+template <class R, int QL, bool DENSE = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
-    int rc = allow_big_lds(fused_step_kernel<R, kMinWaves, QL>, lds_bytes);
+    int rc = allow_big_lds(fused_step_kernel<R, kMinWaves, QL, DENSE>, lds_bytes);
     if (rc) return rc;
-    fused_step_kernel<R, kMinWaves, QL><<<grid, kWG, lds_bytes, s>>>(P);
+    fused_step_kernel<R, kMinWaves, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
     return launch_status();
+}
+
+// alpha > 0: the instances with a run-time quantisation group only
+template <template <int> class RT>
+static int launch_fused_dense(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                              const FusedParams &P) {
+    switch (C) {
+        case kClass0: return launch_fused_one<RT<kClass0>, 0, true>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0, true>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0, true>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0, true>(grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
 }
 
 template <template <int> class RT>
@@ -1832,6 +1962,7 @@ int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
 
 static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream,
                      bool span, double alpha, void *ws, int64_t ws_bytes) {
+    const bool dense = !span && alpha > 0.0;
     if (!tensors || !h || n_tensors < 0) return MA_ERR_ARG;
     for (int i = 0; i < n_tensors; ++i) {
         const int rc = span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h);
@@ -1875,7 +2006,11 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.keep = (float)(1.0 - alpha);
             if (P.L.total > kLdsLimit) return MA_ERR_LDS;
             int rc = 0;
-            if (!span) {
+            if (dense) {
+                rc = h->dtype == MA_BF16
+                         ? launch_fused_dense<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
+                         : launch_fused_dense<RegsF32>(C, (unsigned)items, P.L.total, s, P);
+            } else if (!span) {
                 rc = h->dtype == MA_BF16
                          ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
                          : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
@@ -1935,6 +2070,12 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
 
 int ma_fused_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream) {
     return step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0);
+}
+
+int ma_fused_step_densified(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
+                            double alpha, void *stream) {
+    if (!(alpha > 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
+    return step_impl(tensors, n_tensors, h, stream, false, alpha, nullptr, 0);
 }
 
 int ma_spanning_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {

@@ -56,6 +56,8 @@ def _load():
         "ma_param_update": (ci, [i64, vp, vp, f32, ci, f32, ci, vp]),
         "ma_fused_step": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper), vp]),
         "ma_fused_step_check": (ci, [ctypes.POINTER(MaTensor), ctypes.POINTER(MaHyper)]),
+        "ma_fused_step_densified": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
+                                         ctypes.c_double, vp]),
         "ma_spanning_step": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
                                    ctypes.c_double, vp, ctypes.c_int64, vp]),
         "ma_spanning_step_workspace": (ctypes.c_int64, [ctypes.POINTER(MaTensor), ci,
@@ -74,7 +76,7 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_get_max_floats_for_shared_memory_per_thread_block", "ma_copy_values",
            "ma_zerorize_block_components", "ma_asymm_block_quant", "ma_asymm_block_quant_inv",
            "ma_compute_microadam_update", "ma_block_topk", "ma_block_minmax", "ma_param_update",
-           "ma_fused_step", "ma_fused_step_check", "ma_spanning_step",
+           "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified", "ma_spanning_step",
            "ma_spanning_step_workspace", "ma_spanning_step_check")
 
 

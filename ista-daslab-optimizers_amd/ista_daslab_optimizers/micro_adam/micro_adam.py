@@ -143,7 +143,7 @@ class MicroAdam(torch.optim.Optimizer):
         norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe = 0, 0, 0, 0, 0, 0
         logging_step = self._logging_active() and self.steps % self.log_interval == 0
 
-        fused, spanning = [], []  # (p, st, lr, wd)
+        fused, spanning, dense = [], [], []  # (p, st, lr, wd)
         for group in self.param_groups:
             lr = group['lr']
             wd = group.get('weight_decay', self.weight_decay)
@@ -163,7 +163,7 @@ class MicroAdam(torch.optim.Optimizer):
 
                 route = self._fusable(p, st) if self.use_fused and not logging_step else 0
                 if route:
-                    (fused if route == 1 else spanning).append((p, st, lr, wd))
+                    (fused, spanning, dense)[route - 1].append((p, st, lr, wd))
                     continue
 
                 nqe, ng, nu, ne, sp_u, sp_qe = self.update_step(p, lr, wd, logging_step)
@@ -178,6 +178,8 @@ class MicroAdam(torch.optim.Optimizer):
             self._fused_step(fused)
         if spanning:
             self._fused_step(spanning, spanning=True)
+        if dense:
+            self._fused_step(dense, dense=True)
 
         time_end = time.time()
         elapsed_step = time_end - time_start
@@ -237,7 +239,8 @@ class MicroAdam(torch.optim.Optimizer):
     def _fusable(self, p, st):
         """0: op-by-op route; 1: ma_fused_step (alpha == 0, quantisation blocks inside the top-k
         blocks); 2: ma_spanning_step (0 <= alpha < 1, quantisation blocks at least as long as the
-        top-k blocks).  The conditions are those of include/microadam_hip.h."""
+        top-k blocks); 3: ma_fused_step_densified (as 1 with 0 < alpha < 1).  The conditions are
+        those of include/microadam_hip.h."""
         if not 0 <= self.alpha < 1:
             return 0
         g = p.grad
@@ -251,19 +254,20 @@ class MicroAdam(torch.optim.Optimizer):
             common = (self.m <= _hip.MA_MAX_WINDOW and dbs <= 32768
                       and (d <= self.d_block_size or dbs % 8 == 0))
             route = 0
-            if (common and self.alpha == 0 and 8 <= q <= 512 and (q & (q - 1)) == 0 and d >= q
+            if (common and 8 <= q <= 512 and (q & (q - 1)) == 0 and d >= q
                     and (d <= self.d_block_size or dbs % q == 0)):
-                route = 1
+                route = 1 if self.alpha == 0 else 3
             elif (common and q % 8 == 0 and dbs <= q < (1 << 30)
                   and (q + dbs - 1) // dbs + 1 <= 64):
                 route = 2
             self._route[id(p)] = route
         return route
 
-    def _fused_step(self, items, spanning=False):
+    def _fused_step(self, items, spanning=False, dense=False):
         n = len(items)
-        key = (spanning,) + tuple(id(p) for p, _, _, _ in items)
-        cache = self._fused_cache.get(spanning) if self._fused_cache else None
+        kind = 1 if spanning else 2 if dense else 0
+        key = (kind,) + tuple(id(p) for p, _, _, _ in items)
+        cache = self._fused_cache.get(kind) if self._fused_cache else None
         if cache is None or cache[0] != key:
             arr = (_hip.MaTensor * n)()
             for t, (p, st, _, _) in zip(arr, items):
@@ -272,7 +276,7 @@ class MicroAdam(torch.optim.Optimizer):
             cache = (key, arr)
             if self._fused_cache is None:
                 self._fused_cache = {}
-            self._fused_cache[spanning] = cache
+            self._fused_cache[kind] = cache
         arr = cache[1]
         for t, (p, st, lr, wd) in zip(arr, items):
             t.p = p.data_ptr()
@@ -297,6 +301,11 @@ class MicroAdam(torch.optim.Optimizer):
             h = _hip.MaHyper(self.steps, self.m, _hip.MA_BF16 if dtype == torch.bfloat16 else _hip.MA_F32,
                              self.quant_block_size, self.d_block_size, self.k_init, self.beta1,
                              self.beta2, self.eps)
+            if dense:
+                rc = _hip.lib.ma_fused_step_densified(sub, cnt, ctypes.byref(h), float(self.alpha),
+                                                      _hip.stream_ptr())
+                _hip.check(rc, "ma_fused_step_densified")
+                continue
             if not spanning:
                 rc = _hip.lib.ma_fused_step(sub, cnt, ctypes.byref(h), _hip.stream_ptr())
                 _hip.check(rc, "ma_fused_step")

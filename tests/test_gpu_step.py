@@ -112,6 +112,24 @@ def test_step_spanning_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, 
          expect_route=use_fused)
 
 
+FUSED_DENSIFIED_CASES = [
+    # 0 < alpha < 1 with quantisation blocks inside the top-k blocks: one pass
+    ([20480 * 2 + 4096, 768, 4096], torch.bfloat16, 10, 64, 0.01, 0.5, 0.0, 20480, 12),
+    ([3000, 257, 64, 1024], torch.bfloat16, 4, 64, 0.01, 0.25, 0.1, 1024, 9),
+    ([5000], torch.float32, 3, 64, 0.02, 0.7, 0.0, 2048, 7),
+    ([20480 + 4096], torch.float32, 10, 32, 0.01, 0.1, 0.01, 20480, 12),
+    ([1001, 777], torch.bfloat16, 3, 64, 0.03, 0.5, 0.0, 20480, 5),   # odd d: partial chunks
+]
+
+
+@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
+@pytest.mark.parametrize("sizes,dtype,m,q,k_init,alpha,wd,DB,steps", FUSED_DENSIFIED_CASES)
+def test_step_fused_densified_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps,
+                                    use_fused):
+    _run(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused, zero_step=2,
+         expect_route=use_fused)
+
+
 @pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
 @pytest.mark.parametrize("scale", [1e-36, 3e-38, 1e-39])
 def test_denormal_scale_gradients(oracle, scale, use_fused):
