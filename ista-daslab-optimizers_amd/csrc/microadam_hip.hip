@@ -1475,12 +1475,14 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     const int ti = find_tensor(P, (int)blockIdx.x);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
     auto run = [&](auto &fb) {
-        fb.load_params_window(G);
+        // the parameters and window entries are asked for early where the registers allow it
+        if constexpr (!DENSE) fb.load_params_window(G);
         fb.load_grad_inputs(G);
         fb.dequant(G);
         fb.topk_and_row(G);
         if constexpr (DENSE) {
             fb.quantize_dense(G);
+            fb.load_params_window(G);
             fb.window_stage(G);
             fb.param_stage_dense(G);
         } else {
@@ -1640,10 +1642,14 @@ static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const F
     return launch_status();
 }
 
-// alpha > 0: the instances with a run-time quantisation group only
+// alpha > 0
 template <template <int> class RT>
 static int launch_fused_dense(int C, unsigned grid, int lds_bytes, hipStream_t s,
                               const FusedParams &P) {
+    if (C == kClass2 && P.q_shift == 6)
+        return launch_fused_one<RT<kClass2>, 8, true>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 5)
+        return launch_fused_one<RT<kClass2>, 4, true>(grid, lds_bytes, s, P);
     switch (C) {
         case kClass0: return launch_fused_one<RT<kClass0>, 0, true>(grid, lds_bytes, s, P);
         case kClass1: return launch_fused_one<RT<kClass1>, 0, true>(grid, lds_bytes, s, P);
