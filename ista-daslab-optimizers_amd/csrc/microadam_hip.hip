@@ -502,10 +502,18 @@ struct FusedBlock {
 
     // ---- parameters and the older window rows: requested early, consumed last
     __device__ __forceinline__ void load_params_window(const BlockGeo &G) {
+        load_params(G);
+        load_window(G);
+    }
+
+    __device__ __forceinline__ void load_params(const BlockGeo &G) {
         const int n = FULL ? C * kRound : G.n;
         const elem_t *p = reinterpret_cast<const elem_t *>(G.D.p) + G.e0;
 #pragma unroll
         for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
+    }
+
+    __device__ __forceinline__ void load_window(const BlockGeo &G) {
         const bool fw = fast_window(G);
         const int entries = fw ? P.W.rows * G.kb : 0;
         const float rkb = __builtin_amdgcn_rcpf((float)G.kb);
@@ -1524,9 +1532,10 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             fb.span_store_residual(G, S);
         } else {
             fb.row_in_lds = false;
-            fb.load_params_window(G);
+            fb.load_window(G);
             fb.span_load_residual(G);
             fb.template span_statistics<PASS == 2>(G, S);
+            fb.load_params(G);
             fb.window_stage(G);
             fb.template span_param_stage<PASS == 2>(G, S);
         }
