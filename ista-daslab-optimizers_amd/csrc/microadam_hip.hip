@@ -1141,7 +1141,7 @@ struct FusedBlock {
     }
 
     // min / max over the workgroup of two pairs; every thread gets the result.  Uses the 32
-    // words at kShW1 and two barriers.
+    // words at kShW1 and three barriers.
     __device__ __forceinline__ void wg_minmax2(float (&mn)[2], float (&mx)[2]) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) group_minmax<0>(mn[s2], mx[s2], kWave);
@@ -1160,6 +1160,7 @@ struct FusedBlock {
             mn[1] = fmin_raw(mn[1], __uint_as_float(sh[kShW1 + w * 4 + 2]));
             mx[1] = fmax_raw(mx[1], __uint_as_float(sh[kShW1 + w * 4 + 3]));
         }
+        __syncthreads();  // the words are free again
     }
 
     __device__ __forceinline__ void store_partials(const BlockGeo &G, float (&mn)[2],
@@ -1387,6 +1388,51 @@ struct FusedBlock {
         for (int c = 0; c < C; ++c) graw[c].load(g, chunk_off<C>(wave, c, lane), n, FULL);
     }
 
+    // alpha == 0, second pass: e = Q(r) against the statistics of r, and the statistics arrays
+    __device__ __forceinline__ void span_codes_stage(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        uint8_t *err = D.err + (G.e0 >> 1);
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                const bool second = off >= S.bnd;
+                float x[8], cf[8];
+                graw[c].to_float(x);
+                codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+        }
+        span_store_statistics(G, S);
+    }
+
+    // the block that holds the first element of a quantisation block writes its statistics
+    __device__ __forceinline__ void span_store_statistics(const BlockGeo &G, const Span &S) {
+        if (tid == 0) {
+            if (G.e0 == S.qb0 * (int64_t)P.q_span) {
+                G.D.mn[S.qb0] = (uint16_t)sp2_mn[0];
+                G.D.mx[S.qb0] = (uint16_t)sp2_mx[0];
+            }
+            if (S.bnd != 0x7fffffff) {
+                G.D.mn[S.qb0 + 1] = (uint16_t)sp2_mn[1];
+                G.D.mx[S.qb0 + 1] = (uint16_t)sp2_mx[1];
+            }
+        }
+    }
+
     // DENSE (alpha > 0): p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
     // r2 = rne(0 + keep * d1); e = Q(r2).  Otherwise (alpha == 0): e = Q(r); p += -lr * Adam.
     // Then the statistics arrays.  After window_stage.
@@ -1453,17 +1499,7 @@ struct FusedBlock {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // the block that holds the first element of a quantisation block writes its statistics
-        if (tid == 0) {
-            if (G.e0 == S.qb0 * (int64_t)P.q_span) {
-                D.mn[S.qb0] = (uint16_t)sp2_mn[0];
-                D.mx[S.qb0] = (uint16_t)sp2_mx[0];
-            }
-            if (S.bnd != 0x7fffffff) {
-                D.mn[S.qb0 + 1] = (uint16_t)sp2_mn[1];
-                D.mx[S.qb0 + 1] = (uint16_t)sp2_mx[1];
-            }
-        }
+        span_store_statistics(G, S);
     }
 };
 
@@ -1516,8 +1552,10 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     }
 }
 
-// Two-pass route, see FusedBlock.  PASS 1; then PASS 2 (alpha > 0) or PASS 3 (alpha == 0); one
-// workgroup per block.
+// Two-pass route, see FusedBlock; one workgroup per block.
+//   alpha > 0:  PASS 1 (residual and its extremes), PASS 2 (everything else)
+//   alpha == 0: PASS 4 (PASS 1 and the parameter update, which does not wait for the
+//               statistics), PASS 3 (codes of the residual)
 template <class R, int MIN_WAVES, int PASS>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -1525,19 +1563,27 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + ((int)blockIdx.x - P.t[ti].first_block));
     auto run = [&](auto &fb) {
         const auto S = fb.make_span(G);
-        if constexpr (PASS == 1) {
+        if constexpr (PASS == 1 || PASS == 4) {
             fb.span_load_grad_inputs(G, S);
             fb.span_dequant(G, S);
             fb.topk_and_row(G);
             fb.span_store_residual(G, S);
-        } else {
+            if constexpr (PASS == 4) {
+                fb.load_params_window(G);
+                fb.update(G);
+            }
+        } else if constexpr (PASS == 2) {
             fb.row_in_lds = false;
             fb.load_window(G);
             fb.span_load_residual(G);
-            fb.template span_statistics<PASS == 2>(G, S);
+            fb.template span_statistics<true>(G, S);
             fb.load_params(G);
             fb.window_stage(G);
-            fb.template span_param_stage<PASS == 2>(G, S);
+            fb.template span_param_stage<true>(G, S);
+        } else {
+            fb.span_load_residual(G);
+            fb.template span_statistics<false>(G, S);
+            fb.span_codes_stage(G, S);
         }
     };
     if (G.n == R::kC * kRound) {
@@ -1687,18 +1733,25 @@ template <class R>
 static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
                            const FusedParams &P) {
     int rc;
-    if (pass == 1) {
-        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
-        if (rc) return rc;
-        span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
-    } else if (pass == 2) {
-        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
-        if (rc) return rc;
-        span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
-    } else {
-        rc = allow_big_lds(span_step_kernel<R, kMinWaves, 3>, lds_bytes);
-        if (rc) return rc;
-        span_step_kernel<R, kMinWaves, 3><<<grid, kWG, lds_bytes, s>>>(P);
+    switch (pass) {
+        case 1:
+            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        case 2:
+            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        case 4:
+            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 4>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kMinWaves, 4><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        default:  // needs the kSh* words only
+            span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
+            break;
     }
     return launch_status();
 }
@@ -2031,11 +2084,13 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                          ? launch_fused<RegsBF16>(C, (unsigned)items, P.L.total, s, P)
                          : launch_fused<RegsF32>(C, (unsigned)items, P.L.total, s, P);
             } else {
-                const int second = alpha > 0.0 ? 2 : 3;
-                for (int pass = 1; pass <= second && rc == 0; pass += second - 1)
+                const int passes[2] = {alpha > 0.0 ? 1 : 4, alpha > 0.0 ? 2 : 3};
+                for (int i = 0; i < 2 && rc == 0; ++i) {
+                    const int pass = passes[i];
                     rc = h->dtype == MA_BF16
                              ? launch_span<RegsBF16>(C, pass, (unsigned)items, P.L.total, s, P)
                              : launch_span<RegsF32>(C, pass, (unsigned)items, P.L.total, s, P);
+                }
             }
             count = 0;
             items = 0;
