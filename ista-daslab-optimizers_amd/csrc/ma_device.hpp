@@ -707,7 +707,7 @@ struct WindowView {
     const float *w2;
 };
 
-constexpr int kWindowDepth = 8;
+constexpr int kWindowDepth = 4;
 
 __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, int lo, int hi,
                                                   float *z1, float *z2) {

@@ -234,7 +234,8 @@ struct LdsMap {
     int z_cap;        // entries the window stage's arrays hold
     int sub_len;      // coordinates handled per window pass
     int fast_cap;     // entries the one-pass window stage has room for, 0: none
-    int cell_bytes;   // width of a slot cell: 2, or 4 for fp32 data in the general window stage
+    int cell_bytes;   // width of a slot cell: 2, or 4 for fp32 data in the general window stage;
+                      // 0: no cells, the general window stage updates the parameters range by range
     int total;        // bytes
 };
 constexpr int kMiscBytes = 256;  // the kSh* words at the very start
@@ -480,7 +481,8 @@ struct FusedBlock {
         cell16 = reinterpret_cast<uint16_t *>(lds + P.L.off_slot);
         cell32 = reinterpret_cast<uint32_t *>(lds + P.L.off_slot);
         hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
-        z1 = reinterpret_cast<float *>(lds + P.L.off_union);
+        // without cells the sums of a coordinate range take everything from the cells' place on
+        z1 = reinterpret_cast<float *>(lds + (P.L.cell_bytes == 0 ? P.L.off_slot : P.L.off_union));
         z2 = z1 + P.L.z_cap;
         coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
         tid = threadIdx.x;
@@ -760,8 +762,64 @@ struct FusedBlock {
     //      and p += -lr * u (MA:304).  The slot cells end up holding the update's bits, 0
     //      where no window row names the coordinate.
     __device__ __forceinline__ void update(const BlockGeo &G) {
-        window_stage(G);
-        param_stage(G);
+        if (P.L.cell_bytes == 0) {
+            update_by_ranges(G);
+        } else {
+            window_stage(G);
+            param_stage(G);
+        }
+    }
+
+    // General window stage without coordinate cells: for each coordinate range (a multiple of
+    // 512, so a chunk lies inside one range) the sums, then the Adam direction in place of
+    // z1, then the parameter update of the chunks in the range.
+    __device__ __forceinline__ void update_by_ranges(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        WindowView wv;
+        wv.I = D.I + G.col0;
+        wv.V = D.V + G.col0;
+        wv.k = D.k;
+        wv.rows = P.W.rows;
+        wv.cur_row = row_in_lds ? D.row : -1;
+        wv.cur_idx = sel_idx;
+        wv.cur_val = sel_val;
+        wv.w1 = P.W.w1;
+        wv.w2 = P.W.w2;
+        __syncthreads();  // the LDS of the selection is reused below
+        for (int lo = 0; lo < n; lo += P.L.sub_len) {
+            const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+            window_accumulate(wv, G.kb, lo, hi, z1, z2);
+            for (int c = tid; c < hi - lo; c += kWG) {
+                float u = 0.0f;
+                if (z1[c] != 0.0f || z2[c] != 0.0f)
+                    u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                z1[c] = R::kBF16 ? bf2f(f2bf(u)) : u;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const int off = chunk_off<C>(wave, c, lane);
+                if (off >= lo && off < hi && (FULL || off < n)) {
+                    float pv[8];
+                    praw[c].to_float(pv);
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        // the range may end inside the chunk only at the end of the block
+                        const float u = (FULL || off + e < n) ? z1[off - lo + e] : 0.0f;
+                        if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                        const float prod = neg_lr * u;
+                        pv[e] = pv[e] + prod;
+                    }
+                    store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+                }
+            }
+            __syncthreads();
+        }
+        pt.mark(16);
     }
 
     // The slot cells end up holding the update's bits, 0 where no window row names the
@@ -1599,11 +1657,14 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
 // Host side
 // =============================================================================================
 
+constexpr int kLdsLimit = 160 * 1024;
+
 static inline int align16(int x) { return (x + 15) & ~15; }
 
 // LDS plan for a block kernel: longest block `dbs_max`, most entries per block row `kb_max`,
 // window length m, bytes per element of the data.
-static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_pass = true) {
+static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_pass = true,
+                       bool ranges_update = false) {
     LdsMap L;
     L.off_sel_idx = kMiscBytes;
     L.off_sel_val = L.off_sel_idx + align16(kb_max * 2);
@@ -1614,11 +1675,24 @@ static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_
     const int64_t entries = (int64_t)m * kb_max;
     const bool fast = one_pass && entries <= kEnt * kWG && m <= kFastRows;
     L.cell_bytes = (elem_bytes == 2 || fast) ? 2 : 4;
-    L.off_union = L.off_slot + align16(L.slot_cells * L.cell_bytes);
+    if (!fast && ranges_update) L.cell_bytes = 0;
+    L.off_union = L.off_slot + align16(L.slot_cells * (L.cell_bytes ? L.cell_bytes : 2));
     L.fast_cap = 0;
     if (fast) {
         L.fast_cap = L.z_cap = (int)(entries < 8 ? 8 : entries);
         L.sub_len = L.slot_cells;
+    } else if (L.cell_bytes == 0) {
+        // the sums take the place of the cells and of the selection's histograms: as many
+        // coordinates per range as fit beside a second workgroup on the CU, in units of 512
+        const int room = kLdsLimit / 2 - L.off_slot;
+        const int have = L.off_union + kHistBytes - L.off_slot;
+        int sub = (room > have ? room : have) / 8 / 512 * 512;
+        const int passes = (L.slot_cells + sub - 1) / sub;
+        sub = ((L.slot_cells + passes - 1) / passes + 511) / 512 * 512;  // even them out
+        L.sub_len = L.z_cap = sub;
+        const int zb = 8 * sub;
+        L.total = L.off_slot + align16(zb > have ? zb : have);
+        return L;
     } else {
         L.sub_len = L.slot_cells < 4096 ? L.slot_cells : 4096;
         L.z_cap = L.sub_len;
@@ -1655,7 +1729,6 @@ static int allow_big_lds(K kernel, int bytes) {
                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-constexpr int kLdsLimit = 160 * 1024;
 constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
 // chunks per thread that cover a block of `dbs` elements; 0 if none does
@@ -2066,7 +2139,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             if (count == 0) return 0;
             P.n_tensors = count;
             P.W = W;
-            P.L = plan_lds(dbs_max, kb_max, h->m, elem_bytes);
+            P.L = plan_lds(dbs_max, kb_max, h->m, elem_bytes, true, !span && !dense);
             P.d_block_size = d_block_size;
             P.q_shift = q_shift;
             P.total_items = (int32_t)items;
