@@ -67,10 +67,10 @@ WORKLOADS = {
     "outlier-1.3b": (outlier_1p3b, "bf16", 20, 0.05, 32, 0.0, 1e-3),
     "llama3-8b": (llama3_8b, "bf16", 10, 0.01, 100000, 0.5, 1e-3),
     "plumbing-1m": (lambda: [(1048576,)], "f32", 10, 0.01, 64, 0.0, 1.0),
-    # not a BASELINE configuration: the 7B list with the quantisation block of the reference's
+    # not one of the five benchmark configurations: the 7B list with the quantisation block of the reference's
     # README (quant_block_size=100_000, alpha=0), which takes the two-pass route
     "llama2-7b-q100k": (llama2_7b, "bf16", 10, 0.01, 100000, 0.0, 1e-3),
-    # not a BASELINE configuration either: the 7B list with alpha > 0 and short quantisation blocks
+    # not one of the five either: the 7B list with alpha > 0 and short quantisation blocks
     "llama2-7b-alpha": (llama2_7b, "bf16", 10, 0.01, 64, 0.5, 1e-3),
 }
 
