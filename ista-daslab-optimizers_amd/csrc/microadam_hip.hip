@@ -1491,10 +1491,8 @@ struct FusedBlock {
         }
     }
 
-    // DENSE (alpha > 0): p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
-    // r2 = rne(0 + keep * d1); e = Q(r2).  Otherwise (alpha == 0): e = Q(r); p += -lr * Adam.
-    // Then the statistics arrays.  After window_stage.
-    template <bool DENSE>
+    // alpha > 0, second pass: p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
+    // r2 = rne(0 + keep * d1); e = Q(r2); the statistics arrays.  After window_stage.
     __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
@@ -1514,13 +1512,11 @@ struct FusedBlock {
                 float x[8], cf[8], d1[8];
                 graw[c].to_float(x);
                 codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
-                if (DENSE) {
-                    const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
+                const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
 #pragma unroll
-                    for (int e = 0; e < kChunk; ++e) {
-                        float deq = cf[e] * u;
-                        d1[e] = deq + mnf;
-                    }
+                for (int e = 0; e < kChunk; ++e) {
+                    float deq = cf[e] * u;
+                    d1[e] = deq + mnf;
                 }
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
@@ -1529,20 +1525,15 @@ struct FusedBlock {
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
                     if (apply_decay) pv[e] = to_elem(pv[e] * decay);
-                    float ud = uv[e];
-                    if (DENSE) {
-                        const float add = P.alpha * d1[e];
-                        ud = to_elem(uv[e] + add);
-                    }
+                    const float add = P.alpha * d1[e];
+                    const float ud = to_elem(uv[e] + add);
                     const float prod = neg_lr * ud;
                     pv[e] = pv[e] + prod;
-                    if (DENSE) {
-                        const float keep = P.keep * d1[e];
-                        r2[e] = to_elem(0.0f + keep);
-                    }
+                    const float keep = P.keep * d1[e];
+                    r2[e] = to_elem(0.0f + keep);
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
-                if (DENSE) codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
+                codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
                     if (!FULL && off + e >= n) cf[e] = 0.0f;
@@ -1637,7 +1628,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             fb.template span_statistics<true>(G, S);
             fb.load_params(G);
             fb.window_stage(G);
-            fb.template span_param_stage<true>(G, S);
+            fb.span_param_stage(G, S);
         } else {
             fb.span_load_residual(G);
             fb.template span_statistics<false>(G, S);
