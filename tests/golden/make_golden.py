@@ -22,6 +22,11 @@ CASES = {
     "f32_q64_wd": ([4096], "f32", 3, 64, 0.02, 0.0, 0.01, 2048, 5),
     "bf16_alpha": ([2500, 33], "bf16", 3, 1000, 0.01, 0.5, 0.0, 1024, 5),
     "bf16_block20480": ([20480 + 4096], "bf16", 3, 64, 0.01, 0.0, 0.0, 20480, 4),
+    # quantisation blocks longer than the top-k blocks, without and with alpha
+    "bf16_longq": ([1024 * 5 + 77, 300], "bf16", 4, 2048, 0.02, 0.0, 0.0, 1024, 5),
+    "bf16_longq_alpha": ([1024 * 5 + 77], "bf16", 4, 2048, 0.02, 0.3, 0.0, 1024, 5),
+    "bf16_q64_alpha": ([3000, 1024], "bf16", 3, 64, 0.02, 0.5, 0.01, 1024, 5),
+    "f32_alpha_minus2": ([2000], "f32", 3, 64, 0.02, -2, 0.0, 1024, 4),
 }
 
 
