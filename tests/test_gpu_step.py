@@ -249,3 +249,30 @@ def test_cpu_parameter_is_rejected():
     p.grad = torch.ones(100)
     with pytest.raises(RuntimeError):
         opt.step()
+
+
+def test_unaligned_views_take_the_general_route(oracle):
+    """Parameters and gradients that are views at an odd element offset (not 16-byte aligned)
+    cannot use the vector paths of the fused kernels; the step must still match."""
+    from ista_daslab_optimizers import MicroAdam
+    gen = torch.Generator().manual_seed(11)
+    n, m, q = 5000, 3, 64
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(torch.bfloat16)
+    oparams = [to_np(p0)]
+    oref = oracle.OracleMicroAdam(oparams, m, 1e-3, q, 0.02, 0, d_block_size=2048)
+    pbuf = torch.zeros(n + 8, dtype=torch.bfloat16, device="cuda")
+    pbuf[3:3 + n] = p0.cuda()
+    gp = torch.nn.Parameter(pbuf[3:3 + n])
+    assert gp.data_ptr() % 16 != 0
+    opt = MicroAdam([gp], m=m, lr=1e-3, quant_block_size=q, k_init=0.02)
+    opt.d_block_size = 2048
+    for s in range(5):
+        g = (torch.randn(n, generator=gen) * 1e-2).to(torch.bfloat16)
+        gbuf = torch.zeros(n + 8, dtype=torch.bfloat16, device="cuda")
+        gbuf[1:1 + n] = g.cuda()
+        gp.grad = gbuf[1:1 + n]
+        opt.step()
+        oref.step([to_np(g)])
+        assert opt._fusable(gp, opt.state[gp]) == 0
+        assert_state_equal(opt.state[gp], oref.state[0], f"step {s + 1}")
+        assert np.array_equal(to_np(gp.data), oparams[0])
