@@ -377,13 +377,14 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
     take_eq = need;
 }
 
-// ---- top-k through chunk maxima (bf16, k much smaller than the block) ---------------------------
+// ---- top-k through thread maxima (bf16, k much smaller than the block) -------------------------
 //
-// Every lane keeps only the largest key of each of its 8-element chunks.  If L is the kb-th
-// largest chunk maximum, at least kb chunks hold an element >= L, so the kb-th largest element
-// T satisfies T >= L: every member of the top-k has key >= L.  For k = 1 % of the block about
-// 1.04 k elements pass that test, and the exact top-k (magnitude first, lowest index on ties)
-// is then taken among those few candidates by rank.  The block itself waits in LDS meanwhile.
+// Every thread keeps the largest key of each of its 8-element chunks, and the largest of those.
+// If L is the kb-th largest thread maximum, at least kb threads hold an element >= L, so the
+// kb-th largest element T satisfies T >= L: every member of the top-k has key >= L.  For k = 1 %
+// of the block about 1.3 k elements pass that test (only chunks whose maximum reaches L are
+// looked at again), and the exact top-k (magnitude first, lowest index on ties) is then taken
+// among those few candidates.  The block itself waits in LDS meanwhile.
 
 // largest 15-bit magnitude key among the 8 bf16 values of a chunk
 __device__ __forceinline__ uint32_t chunk_max_key(const uint32_t (&w)[4]) {
@@ -499,8 +500,12 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     __syncthreads();
     pt.mark(1);
     int unused_take, unused_eq;
-    const uint32_t L = select_kth_key15<C>(cmax, 0xffffffffu, kb, hist, sh + kShSel,
-                                           sh + kShNEq, unused_take, unused_eq);
+    // one key per thread: the largest of its chunk maxima
+    uint32_t tmax[1] = {cmax[0]};
+#pragma unroll
+    for (int c = 1; c < C; ++c) tmax[0] = cmax[c] > tmax[0] ? cmax[c] : tmax[0];
+    const uint32_t L = select_kth_key15<1>(tmax, 1u, kb, hist, sh + kShSel, sh + kShNEq,
+                                           unused_take, unused_eq);
     pt.mark(2);
 
     // candidates: every element with key >= L, wave by wave into the wave's own list
