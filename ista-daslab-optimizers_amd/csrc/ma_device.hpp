@@ -318,13 +318,15 @@ __device__ __forceinline__ void launder(R &r) {
 //
 // Finds the key T of the kb-th largest magnitude and how many entries equal to T belong to
 // the top kb (`take_eq` >= 1).  Each pass histograms one digit of the keys that still match
-// the prefix into `hist`, 32 replicated copies per bin so that every lane adds into its own
-// LDS bank whatever the data look like, then scans the bins from the top.
-//   hist: 257*32 words (bin 256 is a discard bin), sh: 8 words.  Ends with a barrier.
+// the prefix into `hist`, 2^copies_log2 replicated copies per bin (32 where the LDS allows it, so
+// that every lane adds into its own bank whatever the data look like), then scans the bins
+// from the top.
+//   hist: 257 << copies_log2 words (bin 256 is a discard bin), sh: 8 words.  Ends with a barrier.
 template <class R>
 __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, uint32_t *sh,
                                                  uint32_t &T, int &take_eq, PhaseTimer &pt,
-                                                 int pt0) {
+                                                 int pt0, int copies_log2) {
+    const int copies = 1 << copies_log2;
     constexpr int kPasses = R::kBF16 ? 2 : 4;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t prefix = 0, pmask = 0;
@@ -335,8 +337,7 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
         const int shift = R::kBF16 ? (pass == 0 ? 7 : 0) : (pass == 3 ? 0 : 23 - 8 * pass);
         const int nb = 1 << bits;
         const uint32_t dm = nb - 1;
-        for (int i = tid; i < nb * kHistCopies / 4; i += kWG)
-            reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+        for (int i = tid; i < (nb + 1) * copies; i += kWG) hist[i] = 0;
         launder(r);
         __syncthreads();
         if (pass < 2) pt.mark(pt0 + 3 * pass);
@@ -347,7 +348,7 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
                 const uint32_t key = r.key(c, e);
                 // keys off the prefix count into a spare bin: cheaper than branching
                 const uint32_t bin = (key & pmask) == prefix ? ((key >> shift) & dm) : 256u;
-                atomicAdd(&hist[(bin << 5) + (lane & 31)], 1u);
+                atomicAdd(&hist[(bin << copies_log2) + (lane & (copies - 1))], 1u);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -357,8 +358,8 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
         const int bin = nb - 1 - tid;
         uint32_t cnt = 0;
         if (bin >= 0) {
-#pragma unroll 8
-            for (int j = 0; j < kHistCopies; ++j) cnt += hist[(bin << 5) + ((j + tid) & 31)];
+            for (int j = 0; j < copies; ++j)
+                cnt += hist[(bin << copies_log2) + ((j + tid) & (copies - 1))];
         }
         uint32_t incl = wg_incl_scan(cnt, sh, lane, wave);
         uint32_t excl = incl - cnt;
@@ -401,7 +402,7 @@ __device__ __forceinline__ uint32_t chunk_max_key(const uint32_t (&w)[4]) {
     return lo > hi ? lo : hi;
 }
 
-constexpr int kSmallCopies = 8;
+constexpr int kSmallCopies = 2;
 constexpr int kSmallHistWords = 2 * 257 * kSmallCopies;  // one histogram per pass
 
 // kb-th largest of the N * 256 keys (15 bits each) held N per thread; 1 <= kb <= N * 256.
@@ -439,9 +440,9 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int bin = 255 - 4 * lane - i;
-                const uint4 a = reinterpret_cast<const uint4 *>(h)[bin * 2];
-                const uint4 b = reinterpret_cast<const uint4 *>(h)[bin * 2 + 1];
-                c[i] = a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
+                c[i] = 0;
+#pragma unroll
+                for (int k = 0; k < kSmallCopies; ++k) c[i] += h[bin * kSmallCopies + k];
                 tot += c[i];
             }
             const uint32_t incl = wave_incl_scan(tot, lane);
@@ -487,8 +488,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     uint32_t *cand = hist + 2 * kSmallHistWords;
     // the histograms of both selections are cleared here, under the one barrier that also
     // covers the parked block
-    for (int i = tid; i < 2 * kSmallHistWords / 4; i += kWG)
-        reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0, 0, 0, 0);
+    for (int i = tid; i < 2 * kSmallHistWords; i += kWG) hist[i] = 0;
     uint32_t cmax[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) {

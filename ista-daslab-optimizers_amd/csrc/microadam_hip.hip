@@ -234,6 +234,8 @@ struct LdsMap {
     int z_cap;        // entries the window stage's arrays hold
     int sub_len;      // coordinates handled per window pass
     int fast_cap;     // entries the one-pass window stage has room for, 0: none
+    int hist_log2;    // log2 of the histogram copies the general selection has room for
+    int compact;      // bf16 one-pass window stage with slots per coordinate instead of lists
     int cell_bytes;   // width of a slot cell: 2, or 4 for fp32 data in the general window stage;
                       // 0: no cells, the general window stage updates the parameters range by range
     int total;        // bytes
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(kWG) void block_topk_kernel(int64_t d, int dbs, int
     uint32_t T;
     int take_eq;
     PhaseTimer pt;
-    select_threshold(r, kb, hist, sh, T, take_eq, pt, 0);
+    select_threshold(r, kb, hist, sh, T, take_eq, pt, 0, L.hist_log2);
     compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 0);
     for (int j = tid; j < kb; j += kWG) {
         const int idx = sel_idx[j];
@@ -646,7 +648,7 @@ struct FusedBlock {
         if (!topk_done) {
             uint32_t T;
             int take_eq;
-            select_threshold(r, kb, hist, sh, T, take_eq, pt, 1);
+            select_threshold(r, kb, hist, sh, T, take_eq, pt, 1, P.L.hist_log2);
             launder(r);
             pt.mark(7);
             compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh, pt, 8);
@@ -883,6 +885,72 @@ struct FusedBlock {
                 entI[i] = tag;
             }
             __syncthreads();
+            if (R::kBF16 && P.L.compact) {
+                // Slots instead of lists.  A coordinate named by one row gets its update from
+                // that entry.  The others are served row by row, rows separated by barriers:
+                // the first row to come (the lowest) takes a slot for the coordinate and marks
+                // the cell with bit 15 and the slot, later rows add into the slot's sums, so
+                // these are formed in row order.  At most half as many slots as entries.
+                float *s1 = z1, *s2 = z2;
+                uint16_t *scoord = coord;
+                uint32_t multi = 0;  // bit i: entry i shares its coordinate
+#pragma unroll
+                for (int i = 0; i < kEnt; ++i) {
+                    const uint32_t tag = entI[i];
+                    if (tag != 0xffffffffu) {
+                        const uint32_t idx = tag & 0xffffu, row = tag >> 16;
+                        // a cell that a lower row has already marked is not a single either
+                        if (cell16[idx] == 1u << row) {
+                            const float v = bf2f(entV[i]);
+                            const float a1 = __uint_as_float(sh[kShW1 + row]) * v;
+                            const float vv = v * v;
+                            const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
+                            const float u =
+                                adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                            cell16[idx] = (uint16_t)f2bf(u);
+                        } else {
+                            multi |= 1u << i;
+                        }
+                    }
+                }
+                for (int r = 0; r < rows; ++r) {
+#pragma unroll
+                    for (int i = 0; i < kEnt; ++i) {
+                        const uint32_t tag = entI[i];
+                        if (((multi >> i) & 1u) != 0 && (tag >> 16) == (uint32_t)r) {
+                            const uint32_t idx = tag & 0xffffu;
+                            const float v = bf2f(entV[i]);
+                            const float a1 = __uint_as_float(sh[kShW1 + r]) * v;
+                            const float vv = v * v;
+                            const float a2 = __uint_as_float(sh[kShW2 + r]) * vv;
+                            const uint32_t c = cell16[idx];
+                            if ((c & 0x8000u) == 0) {
+                                const uint32_t slot = atomicAdd(mcount, 1u);
+                                if (slot < (uint32_t)cap) {
+                                    cell16[idx] = (uint16_t)(0x8000u | slot);
+                                    s1[slot] = 0.0f + a1;
+                                    s2[slot] = 0.0f + a2;
+                                    scoord[slot] = (uint16_t)idx;
+                                }
+                            } else {
+                                const uint32_t slot = c & 0x7fffu;
+                                s1[slot] = s1[slot] + a1;
+                                s2[slot] = s2[slot] + a2;
+                            }
+                        }
+                    }
+                    __syncthreads();
+                }
+                const int used = (int)(*mcount < (uint32_t)cap ? *mcount : (uint32_t)cap);
+                for (int sl = tid; sl < used; sl += kWG) {
+                    const float u = adam_direction(s1[sl], s2[sl], P.W.s1, P.W.s2, P.W.eps);
+                    cell16[scoord[sl]] = (uint16_t)f2bf(u);
+                }
+                __syncthreads();
+                pt.mark(14);
+                pt.mark(15);
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < kEnt; ++i) {
                 const uint32_t tag = entI[i];
@@ -1669,6 +1737,23 @@ static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_
     if (!fast && ranges_update) L.cell_bytes = 0;
     L.off_union = L.off_slot + align16(L.slot_cells * (L.cell_bytes ? L.cell_bytes : 2));
     L.fast_cap = 0;
+    L.hist_log2 = 5;
+    L.compact = 0;
+    if (fast && elem_bytes == 2 && m < kFastRows) {
+        // bf16: coordinates named by several rows get a slot (two sums and the index, 10
+        // bytes) each, at most half as many as there are entries; together with the small
+        // histograms of the fast selection that lets three workgroups share a CU
+        L.compact = 1;
+        L.fast_cap = (int)(entries < 8 ? 8 : entries);
+        L.z_cap = (L.fast_cap + 1) / 2;
+        L.sub_len = L.slot_cells;
+        const int zb = align16(L.z_cap * 10);
+        int u = zb > kFastTopkBytes ? zb : kFastTopkBytes;
+        L.hist_log2 = 0;
+        while ((257 << (L.hist_log2 + 1)) * 4 <= u && L.hist_log2 < 5) ++L.hist_log2;
+        L.total = L.off_union + align16(u);
+        return L;
+    }
     if (fast) {
         L.fast_cap = L.z_cap = (int)(entries < 8 ? 8 : entries);
         L.sub_len = L.slot_cells;
@@ -1720,6 +1805,7 @@ static int allow_big_lds(K kernel, int bytes) {
                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
+constexpr int kMinWavesDense = 3 * kWG / 256;  // three workgroups per CU
 constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
 // chunks per thread that cover a block of `dbs` elements; 0 if none does
@@ -1756,9 +1842,12 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
 
 template <class R, int QL, bool DENSE = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
-    int rc = allow_big_lds(fused_step_kernel<R, kMinWaves, QL, DENSE>, lds_bytes);
+    // bf16 without the densified update fits 80 registers: three workgroups per CU when the
+    // LDS plan allows it as well
+    constexpr int kWaves_ = (R::kBF16 && !DENSE) ? kMinWavesDense : kMinWaves;
+    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE>, lds_bytes);
     if (rc) return rc;
-    fused_step_kernel<R, kMinWaves, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
+    fused_step_kernel<R, kWaves_, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
     return launch_status();
 }
 
