@@ -1805,7 +1805,7 @@ static int allow_big_lds(K kernel, int bytes) {
                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-constexpr int kMinWavesDense = 3 * kWG / 256;  // three workgroups per CU
+constexpr int kWavesThreeWG = 3 * kWG / 256;  // three workgroups per CU
 constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
 // chunks per thread that cover a block of `dbs` elements; 0 if none does
@@ -1844,7 +1844,7 @@ template <class R, int QL, bool DENSE = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // bf16 without the densified update fits 80 registers: three workgroups per CU when the
     // LDS plan allows it as well
-    constexpr int kWaves_ = (R::kBF16 && !DENSE) ? kMinWavesDense : kMinWaves;
+    constexpr int kWaves_ = (R::kBF16 && !DENSE) ? kWavesThreeWG : kMinWaves;
     int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE>, lds_bytes);
     if (rc) return rc;
     fused_step_kernel<R, kWaves_, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
@@ -1885,12 +1885,14 @@ static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, cons
 template <class R>
 static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
                            const FusedParams &P) {
+    // the first pass has the register needs of the fused kernel
+    constexpr int kFirst = R::kBF16 ? kWavesThreeWG : kMinWaves;
     int rc;
     switch (pass) {
         case 1:
-            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 1>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 1>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kMinWaves, 1><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 1><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 2:
             rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
@@ -1898,9 +1900,9 @@ static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s
             span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 4:
-            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 4>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 4>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kMinWaves, 4><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 4><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         default:  // needs the kSh* words only
             span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
