@@ -1844,7 +1844,7 @@ template <class R, int QL, bool DENSE = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // bf16 without the densified update fits 80 registers: three workgroups per CU when the
     // LDS plan allows it as well
-    constexpr int kWaves_ = (R::kBF16 && !DENSE) ? kWavesThreeWG : kMinWaves;
+    constexpr int kWaves_ = R::kBF16 ? kWavesThreeWG : kMinWaves;
     int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE>, lds_bytes);
     if (rc) return rc;
     fused_step_kernel<R, kWaves_, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
@@ -1895,9 +1895,9 @@ static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s
             span_step_kernel<R, kFirst, 1><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 2:
-            rc = allow_big_lds(span_step_kernel<R, kMinWaves, 2>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 2>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kMinWaves, 2><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 2><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 4:
             rc = allow_big_lds(span_step_kernel<R, kFirst, 4>, lds_bytes);
