@@ -166,7 +166,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=None,
                     help="untimed steps; default m + 2, so that the window is full when timing starts")
     ap.add_argument("--workload", default="llama2-7b", choices=sorted(WORKLOADS))
-    ap.add_argument("--grad-sets", type=int, default=3)
+    ap.add_argument("--grad-sets", type=int, default=None,
+                    help="distinct resident gradient sets used in turn; default m + 2 (no gradient "
+                         "recurs inside the window, as when gradients are redrawn every step) or as "
+                         "many as fit in 60 %% of the device memory")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--op-by-op", action="store_true", help="time the unfused route instead")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -196,6 +199,10 @@ def main():
         p.normal_(0, 0.02)
         params.append(torch.nn.Parameter(p))
     n_params = sum(p.numel() for p in params)
+    if args.grad_sets is None:
+        esize = 2 if dtype == "bf16" else 4
+        free = 0.6 * torch.cuda.get_device_properties(dev).total_memory - 3 * esize * n_params
+        args.grad_sets = int(max(1, min(m + 2, free // (esize * n_params))))
     grad_sets = []
     for _ in range(max(1, args.grad_sets)):
         gs = []
@@ -255,6 +262,7 @@ def main():
         "dtype": "f32",  # arithmetic type; storage type of p and g is config.storage
         "data": "synthetic",
         "config": {"workload": args.workload, "storage": dtype, "params": n_params,
+                   "grad_sets": args.grad_sets,
                    "tensors": len(shapes), "m": m,
                    "k_init": k_init, "quant_block_size": q, "alpha": alpha,
                    "d_block_size": opt.d_block_size,

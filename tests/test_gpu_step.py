@@ -276,3 +276,33 @@ def test_unaligned_views_take_the_general_route(oracle):
         assert opt._fusable(gp, opt.state[gp]) == 0
         assert_state_equal(opt.state[gp], oref.state[0], f"step {s + 1}")
         assert np.array_equal(to_np(gp.data), oparams[0])
+
+
+@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
+def test_window_rows_that_name_the_same_coordinates(oracle, use_fused):
+    """Gradients with the same dominant coordinates in every step: every window row names the
+    same coordinates, so almost all window entries share their coordinate with other rows
+    (the reserve path of the one-pass window stage, where the short list overflows)."""
+    from ista_daslab_optimizers import MicroAdam
+    gen = torch.Generator().manual_seed(21)
+    n, m = 20480 * 2 + 4096, 10
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(torch.bfloat16)
+    spikes = torch.randperm(n, generator=gen)[: n // 100]
+    oparams = [to_np(p0)]
+    oref = oracle.OracleMicroAdam(oparams, m, 1e-3, 64, 0.01, 0, d_block_size=20480)
+    gp = torch.nn.Parameter(p0.clone().cuda())
+    opt = MicroAdam([gp], m=m, lr=1e-3, quant_block_size=64, k_init=0.01)
+    opt.use_fused = use_fused
+    for s in range(13):
+        g = torch.randn(n, generator=gen) * 1e-3
+        g[spikes] += torch.sign(torch.randn(spikes.numel(), generator=gen)) * (1.0 + 0.01 * s)
+        g = g.to(torch.bfloat16)
+        gp.grad = g.clone().cuda()
+        opt.step()
+        oref.step([to_np(g)])
+        assert_state_equal(opt.state[gp], oref.state[0], f"step {s + 1}")
+        assert np.array_equal(to_np(gp.data), oparams[0]), f"step {s + 1}"
+    # the window really is that repetitive: the rows of a block name nearly the same coordinates
+    I = opt.state[gp]["I"][:, :205].long()
+    common = sum(len(set(I[0].tolist()) & set(I[r].tolist())) for r in range(1, m)) / (205 * (m - 1))
+    assert common > 0.8, common
