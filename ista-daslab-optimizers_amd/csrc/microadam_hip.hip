@@ -1842,9 +1842,9 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
 
 template <class R, int QL, bool DENSE = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
-    // bf16 without the densified update fits 80 registers: three workgroups per CU when the
-    // LDS plan allows it as well
-    constexpr int kWaves_ = R::kBF16 ? kWavesThreeWG : kMinWaves;
+    // bf16 blocks of up to 20480 elements fit 80 registers and a third of the LDS: three
+    // workgroups per CU
+    constexpr int kWaves_ = (R::kBF16 && R::kC <= kClass2) ? kWavesThreeWG : kMinWaves;
     int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE>, lds_bytes);
     if (rc) return rc;
     fused_step_kernel<R, kWaves_, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
@@ -1886,7 +1886,7 @@ template <class R>
 static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
                            const FusedParams &P) {
     // the first pass has the register needs of the fused kernel
-    constexpr int kFirst = R::kBF16 ? kWavesThreeWG : kMinWaves;
+    constexpr int kFirst = (R::kBF16 && R::kC <= kClass2) ? kWavesThreeWG : kMinWaves;
     int rc;
     switch (pass) {
         case 1:
