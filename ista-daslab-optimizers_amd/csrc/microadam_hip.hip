@@ -802,9 +802,11 @@ struct FusedBlock {
                 z1[c] = R::kBF16 ? bf2f(f2bf(u)) : u;
             }
             __syncthreads();
+            // store addresses formed afresh, as in param_stage
+            const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                const int off = chunk_off<C>(wave, c, lane);
+                const int off = chunk_off<C>(wave2, c, lane2);
                 if (off >= lo && off < hi && (FULL || off < n)) {
                     float pv[8];
                     praw[c].to_float(pv);
@@ -1092,9 +1094,12 @@ struct FusedBlock {
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
         const bool apply_decay = D.apply_decay != 0;
+        // the store addresses are formed afresh: kept from the loads, they would sit in
+        // registers (or in scratch) through the whole window stage
+        const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int off = chunk_off<C>(wave, c, lane);
+            const int off = chunk_off<C>(wave2, c, lane2);
             if (FULL || off < n) {
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
@@ -1205,9 +1210,12 @@ struct FusedBlock {
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
         const bool apply_decay = D.apply_decay != 0;
+        // the store addresses are formed afresh: kept from the loads, they would sit in
+        // registers (or in scratch) through the whole window stage
+        const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int off = chunk_off<C>(wave, c, lane);
+            const int off = chunk_off<C>(wave2, c, lane2);
             if (FULL || off < n) {
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
