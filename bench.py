@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a plain copy of known size; (workload, op_by_op) -> bytes.  The figures and
 # the commands behind them are in profiles/.
-MEASURED_TRAFFIC = {("llama2-7b", False): 53.2e9}  # profiles/fused_step_llama2-7b_hbm_traffic.txt
+MEASURED_TRAFFIC = {("llama2-7b", False): 50.6e9}  # profiles/fused_step_llama2-7b_hbm_traffic.txt
 
 
 def llama2_7b():
