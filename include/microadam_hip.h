@@ -41,6 +41,7 @@ extern "C" {
 
 #define MA_MAX_WINDOW 64 /* largest window length m the kernels take */
 #define MA_MAX_D_BLOCK 32768
+#define MA_MAX_SPARSE_ROWS 4096 /* most window rows the Sparse M-FAC kernels take */
 
 const char *ma_error_string(int code);
 
@@ -198,6 +199,45 @@ int64_t ma_spanning_step_workspace(const ma_tensor *tensors /* host */, int n_te
 /* 0 if ma_spanning_step would accept this tensor, else the MA_ERR_* it would return. */
 int ma_spanning_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */,
                             double alpha);
+
+/* ---- ista_daslab_cuda_sparse_mfac: the kernels that share the window layout -------------- */
+/* Sparse M-FAC (sparse_mfac/sparse_core_mfac_w_ef.py, SC below) keeps its m gradients in the
+ * same I (int16, block-relative) / V layout as MicroAdam's window; its values are bf16 or, with
+ * use_bf16 = False, fp32 (SC:53-58), hence the values_dtype tag.  m_rows is the number of live
+ * rows the caller passes (min(m, steps), SC:192, :212); rows are k entries apart. */
+
+/* SP(blocks, threads, version, d, m, k, d_block_size, k_block_size, g, I, V, out, use_bf16),
+ * SC:188-201: out[i] += sum_j V[i][j] * g[(j / k_block_size) * d_block_size + I[i][j]] for
+ * i < m_rows; the caller zeroes out first (SC:186).  Products and sums in fp32; per top-k
+ * block a partial sum per row goes to the workspace, a second kernel adds them in a fixed
+ * order, so equal inputs give equal bits.  workspace: device memory, 4-byte aligned, at least
+ * ma_sparse_scalar_products_workspace() bytes, contents need not survive the call. */
+int ma_sparse_scalar_products(int64_t d, int64_t m_rows, int64_t k, int64_t d_block_size,
+                              int64_t k_block_size, const void *g, int g_dtype,
+                              const int16_t *indices, const void *values, int values_dtype,
+                              float *out, void *workspace, int64_t workspace_bytes,
+                              void *stream);
+
+/* *bytes = 4 * m_rows * number of top-k blocks.  Host-only. */
+int ma_sparse_scalar_products_workspace(int64_t d, int64_t m_rows, int64_t k,
+                                        int64_t d_block_size, int64_t k_block_size,
+                                        int64_t *bytes /* host */);
+
+/* LCG(blocks, threads, version, d, m, k, d_block_size, k_block_size, M, I, V, out, use_bf16),
+ * SC:208-221: out[(j / k_block_size) * d_block_size + I[i][j]] += coef[i] * V[i][j] for
+ * i < m_rows; the caller zeroes out first (SC:206).  Per coordinate the terms fl(coef[i] * v)
+ * are added in fp32 in increasing row order, and the sum is added to out with one rounding
+ * into out_dtype. */
+int ma_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d_block_size,
+                                 int64_t k_block_size, const float *coef,
+                                 const int16_t *indices, const void *values, int values_dtype,
+                                 void *out, int out_dtype, void *stream);
+
+/* ma_copy_values with the window values in values_dtype (SC:105-124 with use_bf16 = False keeps
+ * fp32 values); dtype is the dense vector's type as in ma_copy_values. */
+int ma_copy_values_typed(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
+                         const int16_t *indices, const void *inp, void *out, int direction,
+                         int dtype, int values_dtype, void *stream);
 
 #ifdef __cplusplus
 }

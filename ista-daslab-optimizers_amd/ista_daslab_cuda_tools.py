@@ -25,11 +25,19 @@ def copy_values(d, k, d_block_size, k_block_size, indices, inp, out, direction):
     sparse = out if direction == 1 else inp
     if indices.numel() < k or sparse.numel() < k or dense.numel() < d:
         raise RuntimeError("copy_values: tensor shorter than d / k")
-    _hip.dev_ptr(sparse, torch.bfloat16, "values")
-    rc = _hip.lib.ma_copy_values(d, k, d_block_size, k_block_size,
-                                 _hip.dev_ptr(indices, torch.int16, "indices"),
-                                 _hip.dev_ptr(inp, None, "inp"), _hip.dev_ptr(out, None, "out"),
-                                 int(direction), _hip.dtype_tag(dense), _hip.stream_ptr())
+    if sparse.dtype == torch.bfloat16:
+        rc = _hip.lib.ma_copy_values(d, k, d_block_size, k_block_size,
+                                     _hip.dev_ptr(indices, torch.int16, "indices"),
+                                     _hip.dev_ptr(inp, None, "inp"),
+                                     _hip.dev_ptr(out, None, "out"), int(direction),
+                                     _hip.dtype_tag(dense), _hip.stream_ptr())
+    else:  # Sparse M-FAC with use_bf16 = False keeps fp32 values
+        rc = _hip.lib.ma_copy_values_typed(d, k, d_block_size, k_block_size,
+                                           _hip.dev_ptr(indices, torch.int16, "indices"),
+                                           _hip.dev_ptr(inp, None, "inp"),
+                                           _hip.dev_ptr(out, None, "out"), int(direction),
+                                           _hip.dtype_tag(dense), _hip.dtype_tag(sparse),
+                                           _hip.stream_ptr())
     _hip.check(rc, "copy_values")
 
 

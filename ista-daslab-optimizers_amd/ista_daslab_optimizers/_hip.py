@@ -64,6 +64,13 @@ def _load():
                                                          ctypes.POINTER(MaHyper)]),
         "ma_spanning_step_check": (ci, [ctypes.POINTER(MaTensor), ctypes.POINTER(MaHyper),
                                          ctypes.c_double]),
+        "ma_sparse_scalar_products": (ci, [i64, i64, i64, i64, i64, vp, ci, vp, vp, ci, vp, vp,
+                                           i64, vp]),
+        "ma_sparse_scalar_products_workspace": (ci, [i64, i64, i64, i64, i64,
+                                                     ctypes.POINTER(ctypes.c_int64)]),
+        "ma_sparse_linear_combination": (ci, [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp, ci,
+                                              vp]),
+        "ma_copy_values_typed": (ci, [i64, i64, i64, i64, vp, vp, vp, ci, ci, ci, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -77,7 +84,9 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_zerorize_block_components", "ma_asymm_block_quant", "ma_asymm_block_quant_inv",
            "ma_compute_microadam_update", "ma_block_topk", "ma_block_minmax", "ma_param_update",
            "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified", "ma_spanning_step",
-           "ma_spanning_step_workspace", "ma_spanning_step_check")
+           "ma_spanning_step_workspace", "ma_spanning_step_check", "ma_sparse_scalar_products",
+           "ma_sparse_scalar_products_workspace", "ma_sparse_linear_combination",
+           "ma_copy_values_typed")
 
 
 def error_string(code):

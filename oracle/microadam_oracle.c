@@ -447,3 +447,48 @@ int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t 
     }
     return 0;
 }
+
+/* ---- Sparse M-FAC's two window kernels (same I / V layout) ---------------- */
+
+/* ista_daslab_cuda_sparse_mfac.SP, sparse_mfac/sparse_core_mfac_w_ef.py:185-203: the scalar
+ * product of every live window row with the dense vector g,
+ *   out[i] += sum_j V[i][j] * g[blk(j)*DB + I[i][j]],   i < m_rows (= min(m, steps), :192).
+ * The caller zeroes out first (:186).  The order of the sum is not part of the contract (the
+ * device adds per-block partial sums); the oracle accumulates in double so that an fp32
+ * result can be checked against it with a bound on the rounding of the sum alone. */
+void ora_sparse_scalar_products(int64_t d, int64_t m_rows, int64_t k, int64_t d_block_size,
+                                int64_t k_block_size, const void *g, int g_dtype,
+                                const int16_t *indices, const void *values, int v_dtype,
+                                double *out) {
+    (void)d;
+    for (int64_t i = 0; i < m_rows; ++i) {
+        double s = 0.0;
+        for (int64_t j = 0; j < k; ++j) {
+            int64_t pos = (j / k_block_size) * d_block_size + indices[i * k + j];
+            /* the product of two fp32 values is exact in double */
+            s += (double)ld(values, i * k + j, v_dtype) * (double)ld(g, pos, g_dtype);
+        }
+        out[i] += s;
+    }
+}
+
+/* ista_daslab_cuda_sparse_mfac.LCG, sparse_core_mfac_w_ef.py:205-221: the linear combination
+ * of the live window rows with coefficients c (fp32, :167 `M`),
+ *   out[blk(j)*DB + I[i][j]] += c[i] * V[i][j],   i < m_rows.
+ * The caller zeroes out first (:206).  Frozen here: per coordinate the terms fl(c[i] * v) are
+ * added in fp32 in increasing row order (no fused multiply-add), and the sum is added to out
+ * with one rounding into out's type. */
+void ora_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d_block_size,
+                                   int64_t k_block_size, const float *coef,
+                                   const int16_t *indices, const void *values, int v_dtype,
+                                   void *out, int out_dtype) {
+    float *acc = (float *)calloc((size_t)d, sizeof(float));
+    for (int64_t i = 0; i < m_rows; ++i)
+        for (int64_t j = 0; j < k; ++j) {
+            int64_t pos = (j / k_block_size) * d_block_size + indices[i * k + j];
+            float term = coef[i] * ld(values, i * k + j, v_dtype);
+            acc[pos] = acc[pos] + term;
+        }
+    for (int64_t i = 0; i < d; ++i) st(out, i, out_dtype, ld(out, i, out_dtype) + acc[i]);
+    free(acc);
+}

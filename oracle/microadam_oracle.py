@@ -76,6 +76,9 @@ def lib():
         L.ora_update_step.argtypes = [ctypes.POINTER(_Hyper), vp, vp, ci, i64,
                                       ctypes.POINTER(i64), vp, vp, vp, vp, vp]
         L.ora_update_step.restype = ci
+        L.ora_sparse_scalar_products.argtypes = [i64, i64, i64, i64, i64, vp, ci, vp, vp, ci, vp]
+        L.ora_sparse_linear_combination.argtypes = [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp,
+                                                    ci]
         _lib = L
     return _lib
 
@@ -172,6 +175,23 @@ def weight_decay(p, factor):
 
 def param_update(p, u, neg_lr):
     lib().ora_param_update(p.size, _ptr(p), _ptr(u), float(neg_lr), dtype_tag(p), dtype_tag(u))
+
+
+def sparse_scalar_products(d, m_rows, k, d_block_size, k_block_size, g, indices, values, out):
+    """out (float64, length >= m_rows) += scalar products of the window rows with g."""
+    assert out.dtype == np.float64
+    lib().ora_sparse_scalar_products(d, m_rows, k, d_block_size, k_block_size, _ptr(g),
+                                     dtype_tag(g), _ptr(indices), _ptr(values), dtype_tag(values),
+                                     _ptr(out))
+
+
+def sparse_linear_combination(d, m_rows, k, d_block_size, k_block_size, coef, indices, values,
+                              out):
+    """out += sum_i coef[i] * (window row i scattered to length d)."""
+    assert coef.dtype == np.float32
+    lib().ora_sparse_linear_combination(d, m_rows, k, d_block_size, k_block_size, _ptr(coef),
+                                        _ptr(indices), _ptr(values), dtype_tag(values), _ptr(out),
+                                        dtype_tag(out))
 
 
 def unpack_codes(xq, d):

@@ -463,3 +463,102 @@ def test_error_feedback_invariant(oracle):
             rest = np.delete(blk_a, sel)
             assert blk_a[sel].min() >= rest.max()
         prev = deq
+
+
+# ---- Sparse M-FAC's window kernels: scalar products and linear combination -----------------
+
+def _random_window(rng, d, dbs, k_init, m, values_f32):
+    """A window in MicroAdam's layout whose rows name distinct coordinates per top-k block."""
+    import math
+    full, tail0 = d // dbs, (d // dbs) * dbs
+    if d < dbs:
+        full, tail0 = 1, d  # tools.py:85-92
+    kb = math.ceil(min(dbs, d) * k_init)
+    lens = [min(dbs, d)] * full + ([d - tail0] if tail0 < d else [])
+    kbs = [kb] * full + ([math.ceil((d - tail0) * k_init)] if tail0 < d else [])
+    k = sum(kbs)
+    I = np.zeros((m, k), dtype=np.int16)
+    for r in range(m):
+        col = 0
+        for ln, kk in zip(lens, kbs):
+            I[r, col:col + kk] = rng.permutation(ln)[:kk]
+            col += kk
+    Vf = rng.standard_normal((m, k)).astype(np.float32)
+    return I, Vf, k, kb
+
+
+def _dense_rows(I, Vf, d, dbs, kb):
+    """The window as a dense [m, d] float64 matrix (numpy fancy indexing, no oracle code)."""
+    m, k = I.shape
+    pos = (np.arange(k) // kb) * dbs + I.astype(np.int64)
+    G = np.zeros((m, d))
+    G[np.arange(m)[:, None], pos] = Vf
+    return G
+
+
+@pytest.mark.parametrize("values_f32", [False, True])
+@pytest.mark.parametrize("d,dbs,k_init", [(1000, 256, 0.05), (4096, 512, 0.01), (300, 512, 0.1),
+                                          (2048 + 7, 1024, 0.02)])
+def test_sparse_scalar_products_equal_dense_matvec(oracle, values_f32, d, dbs, k_init):
+    rng = np.random.default_rng(d)
+    m = 6
+    I, Vf, k, kb = _random_window(rng, d, dbs, k_init, m, values_f32)
+    V = Vf if values_f32 else oracle.f32_to_bf16(Vf)
+    Vw = Vf if values_f32 else oracle.bf16_to_f32(V)
+    gf = rng.standard_normal(d).astype(np.float32)
+    g = gf if values_f32 else oracle.f32_to_bf16(gf)
+    gw = gf if values_f32 else oracle.bf16_to_f32(g)
+    rows = 4  # the last two rows of the window are not live
+    out = np.full(m, 0.5)
+    oracle.sparse_scalar_products(d, rows, k, dbs, kb, g, I, V, out)
+    want = _dense_rows(I, Vw, d, dbs, kb) @ gw.astype(np.float64)
+    assert np.allclose(out[:rows], 0.5 + want[:rows], rtol=1e-12, atol=1e-12)
+    assert np.all(out[rows:] == 0.5)
+
+
+@pytest.mark.parametrize("out_f32", [False, True])
+@pytest.mark.parametrize("d,dbs,k_init", [(1000, 256, 0.05), (300, 512, 0.1), (2048 + 7, 1024, 0.5)])
+def test_sparse_linear_combination_equals_dense_combination(oracle, out_f32, d, dbs, k_init):
+    rng = np.random.default_rng(d + 1)
+    m = 7
+    I, Vf, k, kb = _random_window(rng, d, dbs, k_init, m, True)
+    V = oracle.f32_to_bf16(Vf)
+    Vw = oracle.bf16_to_f32(V)
+    coef = rng.standard_normal(m).astype(np.float32)
+    rows = 5
+    out = np.zeros(d, dtype=np.float32) if out_f32 else np.zeros(d, dtype=np.uint16)
+    oracle.sparse_linear_combination(d, rows, k, dbs, kb, coef, I, V, out)
+    got = out if out_f32 else oracle.bf16_to_f32(out)
+    G = _dense_rows(I, Vw, d, dbs, kb)
+    want = coef[:rows].astype(np.float64) @ G[:rows]
+    scale = np.abs(coef[:rows]).astype(np.float64) @ np.abs(G[:rows])
+    tol = (2.0 ** -22 if out_f32 else 2.0 ** -8) * scale + 1e-30
+    assert np.all(np.abs(got - want) <= tol)
+    assert np.all(got[scale == 0] == 0)
+
+
+def test_sparse_linear_combination_special_cases(oracle):
+    """One row with coefficient 1 is copy_values k2d; disjoint rows give the exact products;
+    the result is added to what out holds."""
+    rng = np.random.default_rng(5)
+    d, dbs, m = 1536, 512, 3
+    I, Vf, k, kb = _random_window(rng, d, dbs, 0.03, m, True)
+    V = oracle.f32_to_bf16(Vf)
+    out = np.zeros(d, dtype=np.uint16)
+    oracle.sparse_linear_combination(d, 1, k, dbs, kb, np.ones(1, np.float32), I, V, out)
+    scat = np.zeros(d, dtype=np.uint16)
+    oracle.copy_values(d, k, dbs, kb, I[0], V[0], scat, 0)
+    assert np.array_equal(out, scat)
+    # rows on disjoint coordinates: every touched coordinate is one product, rounded once
+    I2 = I.copy()
+    for b in range(d // dbs):
+        perm = rng.permutation(dbs)[:m * kb].reshape(m, kb)
+        I2[:, b * kb:(b + 1) * kb] = perm
+    coef = np.array([0.5, -3.0, 1.25], dtype=np.float32)
+    out = np.full(d, 2.0, dtype=np.float32)
+    oracle.sparse_linear_combination(d, m, k, dbs, kb, coef, I2, V, out)
+    want = np.full(d, 2.0, dtype=np.float32)
+    pos = (np.arange(k) // kb) * dbs + I2.astype(np.int64)
+    for r in range(m):
+        want[pos[r]] = np.float32(2.0) + coef[r] * oracle.bf16_to_f32(V[r])
+    assert np.array_equal(out, want)
