@@ -159,13 +159,103 @@ def route_label(opt, params):
     return next(iter(counts)) if len(counts) == 1 else counts
 
 
+def bench_sparse_window(args):
+    """Sparse M-FAC's two kernels over the shared window layout at a ResNet-50-sized vector:
+    a step is SP (scalar products of the m rows with a dense vector) followed by out.zero_() and
+    LCG (linear combination of the rows), as in sparse_core_mfac_w_ef.py:185-226."""
+    import math
+    import torch
+    import ista_daslab_cuda_sparse_mfac as smf
+    from ista_daslab_optimizers import _hip
+
+    d, dbs, m, k_init = 25_557_032, 20480, 1024, 0.01
+    dev = torch.device("cuda:0")
+    kb = math.ceil(dbs * k_init)
+    tail = d - (d // dbs) * dbs
+    k_few = math.ceil(tail * k_init) if tail else 0
+    k = (d // dbs) * kb + k_few
+    gen = torch.Generator(device=dev).manual_seed(0)
+    I = torch.zeros(m, k, dtype=torch.int16, device=dev)
+    V = torch.zeros(m, k, dtype=torch.bfloat16, device=dev)
+    for r in range(m):  # rows as the optimizer makes them: block top-k of a dense vector
+        x = torch.randn(d, generator=gen, device=dev).to(torch.bfloat16)
+        _hip.check(_hip.lib.ma_block_topk(d, dbs, kb, k_few, _hip.dev_ptr(x), _hip.dev_ptr(I[r]),
+                                          _hip.dev_ptr(V[r]), 0, _hip.MA_BF16, _hip.stream_ptr()),
+                   "block_topk")
+    g = torch.randn(d, generator=gen, device=dev).to(torch.bfloat16)
+    coef = torch.randn(m, generator=gen, device=dev)
+    dots = torch.zeros(m, dtype=torch.float32, device=dev)
+    out = torch.zeros(d, dtype=torch.bfloat16, device=dev)
+    warmup = 3 if args.warmup is None else args.warmup
+
+    def one_step(events=None):
+        dots.zero_()
+        if events:
+            events[0].record()
+        smf.SP(0, 0, 23, d, m, k, dbs, kb, g, I, V, dots, 1)
+        if events:
+            events[1].record()
+        out.zero_()
+        if events:
+            events[2].record()
+        smf.LCG(0, 0, 51, d, m, k, dbs, kb, coef, I, V, out, 1)
+        if events:
+            events[3].record()
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        one_step(ev[i])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    sp_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    lcg_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
+    window_bytes = m * k * 4
+    sp_bytes = window_bytes + 2 * d + 4 * m        # window, g, out
+    lcg_bytes = window_bytes + 4 * d + 4 * m       # window, out read and written, coefficients
+    achieved = (sp_bytes + lcg_bytes) / ((sp_ms + lcg_ms) * 1e-3) / 1e9
+    res = {
+        "metric": "Sparse M-FAC window kernels, SP + LCG (params/s)",
+        "value": d / (ms_per_step * 1e-3), "unit": "params/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "storage": "bf16", "params": d, "m": m,
+                   "k_init": k_init, "d_block_size": dbs, "k": k},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "sp_ms": sp_ms, "sp_gbs": sp_bytes / (sp_ms * 1e-3) / 1e9,
+                     "lcg_ms": lcg_ms, "lcg_gbs": lcg_bytes / (lcg_ms * 1e-3) / 1e9},
+    }
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import numpy as np
+        import microadam_oracle as oracle
+        rows = 32
+        In = I[:rows].cpu().numpy()
+        Vn = V[:rows].cpu().view(torch.int16).numpy().view(np.uint16)
+        gn = g.cpu().view(torch.int16).numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        oracle.sparse_scalar_products(d, rows, k, dbs, kb, gn, In, Vn, np.zeros(rows))
+        oracle.sparse_linear_combination(d, rows, k, dbs, kb, coef[:rows].cpu().numpy(), In, Vn,
+                                         np.zeros(d, dtype=np.uint16))
+        cpu_s = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": d / (cpu_s * m / rows), "unit": "params/s", "cores": 1,
+                               "kind": "port",
+                               "sample": f"{rows} of the {m} window rows, time scaled by {m // rows}"}
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=None,
                     help="untimed steps; default m + 2, so that the window is full when timing starts")
-    ap.add_argument("--workload", default="llama2-7b", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama2-7b",
+                    choices=sorted(WORKLOADS) + ["sparse-mfac-resnet50"])
     ap.add_argument("--grad-sets", type=int, default=None,
                     help="distinct resident gradient sets used in turn; default m + 2 (no gradient "
                          "recurs inside the window, as when gradients are redrawn every step) or as "
@@ -180,6 +270,9 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
+
+    if args.workload == "sparse-mfac-resnet50":
+        return bench_sparse_window(args)
 
     import torch
     from ista_daslab_optimizers import MicroAdam

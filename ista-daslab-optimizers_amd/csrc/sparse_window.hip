@@ -17,9 +17,7 @@ namespace ma {
 namespace {
 
 constexpr int kLdsBytes = 160 * 1024;
-constexpr int kSlots = 8;              // window entries a thread holds per batch
-constexpr int kBatch = kSlots * kWG;   // entries per batch of whole rows
-constexpr int kBatchRows = 32;         // rows per batch at most
+constexpr int kBatchRows = 16;         // rows the linear combination requests ahead
 constexpr int kDotUnroll = 4;          // entries a lane requests ahead in the scalar products
 
 __device__ __forceinline__ float widen(float x) { return x; }
@@ -70,34 +68,53 @@ __global__ __launch_bounds__(kWG) void sparse_dot_kernel(int64_t d, int dbs, int
     for (int i = staged + tid; i < S.len; i += kWG) gl[i] = src[i];
     __syncthreads();
 
-    for (int r = wave; r < m_rows; r += kWG / 64) {
-        const int16_t *Ir = I + (int64_t)r * k + S.col0;
-        const TV *Vr = V + (int64_t)r * k + S.col0;
-        float acc = 0.0f;
+    // the workgroups of one block (gridDim.y of them) share its rows; a wave takes two rows at
+    // a time so that both rows' entries are in flight together
+    constexpr int kWaves = kWG / 64;
+    const int per = (m_rows + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int row_lo = (int)blockIdx.y * per;
+    const int row_hi = row_lo + per < m_rows ? row_lo + per : m_rows;
+    for (int r = row_lo + wave; r < row_hi; r += 2 * kWaves) {
+        const int r2 = r + kWaves;
+        const bool two = r2 < row_hi;
+        const int64_t atA = (int64_t)r * k + S.col0, atB = (int64_t)(two ? r2 : r) * k + S.col0;
+        float accA = 0.0f, accB = 0.0f;
         for (int j0 = 0; j0 < S.kb; j0 += 64 * kDotUnroll) {
-            int ix[kDotUnroll];
-            TV vv[kDotUnroll];
+            int ixA[kDotUnroll], ixB[kDotUnroll];
+            TV vA[kDotUnroll], vB[kDotUnroll];
 #pragma unroll
             for (int u = 0; u < kDotUnroll; ++u) {
                 const int j = j0 + u * 64 + lane;
-                ix[u] = -1;
-                vv[u] = (TV)0;
+                ixA[u] = ixB[u] = -1;
+                vA[u] = vB[u] = (TV)0;
                 if (j < S.kb) {
-                    ix[u] = Ir[j];
-                    vv[u] = Vr[j];
+                    ixA[u] = I[atA + j];
+                    vA[u] = V[atA + j];
+                    if (two) {
+                        ixB[u] = I[atB + j];
+                        vB[u] = V[atB + j];
+                    }
                 }
             }
 #pragma unroll
-            for (int u = 0; u < kDotUnroll; ++u)
-                if ((unsigned)ix[u] < (unsigned)S.len) acc += widen(vv[u]) * widen(gl[ix[u]]);
+            for (int u = 0; u < kDotUnroll; ++u) {
+                if ((unsigned)ixA[u] < (unsigned)S.len) accA += widen(vA[u]) * widen(gl[ixA[u]]);
+                if ((unsigned)ixB[u] < (unsigned)S.len) accB += widen(vB[u]) * widen(gl[ixB[u]]);
+            }
         }
 #pragma unroll
-        for (int s = 32; s > 0; s >>= 1) acc += __shfl_xor(acc, s, 64);
-        if (lane == 0) rowsum[r] = acc;
+        for (int s = 32; s > 0; s >>= 1) {
+            accA += __shfl_xor(accA, s, 64);
+            accB += __shfl_xor(accB, s, 64);
+        }
+        if (lane == 0) {
+            rowsum[r] = accA;
+            if (two) rowsum[r2] = accB;
+        }
     }
     __syncthreads();
     float *dst = partial + (int64_t)blockIdx.x * m_rows;
-    for (int r = tid; r < m_rows; r += kWG) dst[r] = rowsum[r];
+    for (int r = row_lo + tid; r < row_hi; r += kWG) dst[r] = rowsum[r];
 }
 
 // out[r] += sum over blocks of partial[b][r]: a wave per row, lane l adds blocks l, l + 64, ...
@@ -118,8 +135,8 @@ __global__ __launch_bounds__(kWG) void sparse_dot_reduce_kernel(const float *par
 // ---- linear combination ---------------------------------------------------------------------
 // acc[c] (fp32, LDS) takes the terms coef[r] * V[r][j] of the block's coordinates row by row in
 // increasing r: the entries of one row name distinct coordinates, so a row is applied without
-// atomics, and a barrier separates rows.  Whole rows are fetched in batches of up to kBatch
-// entries, the next batch requested before the current one is applied.
+// atomics, and a barrier separates rows.  With at most 512 entries per row a thread holds one
+// column of kBatchRows rows, the next batch requested before the current one is applied.
 template <typename TO, typename TV>
 __global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs, int kbs,
                                                              int64_t k, int m_rows,
@@ -132,51 +149,41 @@ __global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs,
     for (int i = tid; i < S.len; i += kWG) acc[i] = 0.0f;
     __syncthreads();
 
-    if (S.kb <= kBatch) {
-        int rb = kBatch / S.kb;
-        rb = rb > kBatchRows ? kBatchRows : rb;
-        // slot n of this thread is entry jj[n] of the batch's row rr[n] (rr = rb: unused)
-        int rr[kSlots], jj[kSlots];
-#pragma unroll
-        for (int n = 0; n < kSlots; ++n) {
-            const int e = tid + n * kWG;
-            const int row = e / S.kb;
-            rr[n] = row < rb ? row : rb;
-            jj[n] = e - row * S.kb;
-        }
-        int nix[kSlots];
-        float nval[kSlots], ncoef[kSlots];
+    if (S.kb <= kWG) {
+        // thread tid holds column tid of kBatchRows consecutive rows.  Requests are
+        // unconditional (row and column clamped into the window) and their results stay as
+        // loaded until they are applied, so that all of a batch is in flight at once.
+        const bool mine = tid < S.kb;
+        const int16_t *Ic = I + S.col0 + (mine ? tid : 0);
+        const TV *Vc = V + S.col0 + (mine ? tid : 0);
+        int nix[kBatchRows];
+        TV nraw[kBatchRows];
+        float ncoef[kBatchRows];
         auto request = [&](int r0) {
 #pragma unroll
-            for (int n = 0; n < kSlots; ++n) {
-                const int row = r0 + rr[n];
-                nix[n] = -1;
-                nval[n] = 0.0f;
-                ncoef[n] = 0.0f;
-                if (rr[n] < rb && row < m_rows) {
-                    const int64_t at = (int64_t)row * k + S.col0 + jj[n];
-                    nix[n] = I[at];
-                    nval[n] = widen(V[at]);
-                    ncoef[n] = coef[row];
-                }
+            for (int u = 0; u < kBatchRows; ++u) {
+                const int row = r0 + u < m_rows ? r0 + u : m_rows - 1;
+                nix[u] = Ic[(int64_t)row * k];
+                nraw[u] = Vc[(int64_t)row * k];
+                ncoef[u] = coef[row];
             }
         };
         request(0);
-        for (int r0 = 0; r0 < m_rows; r0 += rb) {
-            int ix[kSlots];
-            float term[kSlots];
+        for (int r0 = 0; r0 < m_rows; r0 += kBatchRows) {
+            int ix[kBatchRows];
+            float term[kBatchRows];
 #pragma unroll
-            for (int n = 0; n < kSlots; ++n) {
-                ix[n] = (unsigned)nix[n] < (unsigned)S.len ? nix[n] : -1;
-                term[n] = ncoef[n] * nval[n];
+            for (int u = 0; u < kBatchRows; ++u) {
+                ix[u] = (mine && (unsigned)nix[u] < (unsigned)S.len) ? nix[u] : -1;
+                term[u] = ncoef[u] * widen(nraw[u]);
             }
-            if (r0 + rb < m_rows) request(r0 + rb);
-            const int rows = (m_rows - r0) < rb ? (m_rows - r0) : rb;
-            for (int r = 0; r < rows; ++r) {
+            if (r0 + kBatchRows < m_rows) request(r0 + kBatchRows);
 #pragma unroll
-                for (int n = 0; n < kSlots; ++n)
-                    if (rr[n] == r && ix[n] >= 0) acc[ix[n]] = acc[ix[n]] + term[n];
-                __syncthreads();
+            for (int u = 0; u < kBatchRows; ++u) {
+                if (r0 + u < m_rows) {
+                    if (ix[u] >= 0) acc[ix[u]] = acc[ix[u]] + term[u];
+                    __syncthreads();
+                }
             }
         }
     } else {
@@ -274,9 +281,13 @@ int ma_sparse_scalar_products(int64_t d, int64_t m_rows, int64_t k, int64_t d_bl
     if (lds > kLdsBytes) return MA_ERR_LDS;
     hipStream_t s = (hipStream_t)stream;
     float *partial = (float *)workspace;
+    // enough workgroups to fill the CUs several times over, at least 64 rows each
+    int64_t gy = (4096 + nblocks - 1) / nblocks, gy_max = m_rows / 64;
+    gy = gy > gy_max ? gy_max : gy;
+    gy = gy < 1 ? 1 : gy;
 #define CALL(TG, TV)                                                                            \
     if ((rc = allow_lds(sparse_dot_kernel<TG, TV>, lds))) return rc;                            \
-    sparse_dot_kernel<TG, TV><<<(unsigned)nblocks, kWG, lds, s>>>(                              \
+    sparse_dot_kernel<TG, TV><<<dim3((unsigned)nblocks, gy), kWG, lds, s>>>(                         \
         d, (int)d_block_size, (int)k_block_size, k, (int)m_rows, (const TG *)g, indices,        \
         (const TV *)values, partial);
     MA_DISPATCH2(g_dtype, values_dtype, CALL)
