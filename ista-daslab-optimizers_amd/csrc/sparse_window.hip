@@ -137,8 +137,8 @@ __global__ __launch_bounds__(kWG) void sparse_dot_reduce_kernel(const float *par
 // increasing r: the entries of one row name distinct coordinates, so a row is applied without
 // atomics, and a barrier separates rows.  With at most 512 entries per row a thread holds one
 // column of kBatchRows rows, the next batch requested before the current one is applied.
-template <typename TO, typename TV>
-__global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs, int kbs,
+template <typename TO, typename TV, int WG>
+__global__ __launch_bounds__(WG) void sparse_combine_kernel(int64_t d, int dbs, int kbs,
                                                              int64_t k, int m_rows,
                                                              const float *coef, const int16_t *I,
                                                              const TV *V, TO *out) {
@@ -146,10 +146,10 @@ __global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs,
     float *acc = (float *)lds_raw;
     const BlockSpan S = block_span(d, dbs, kbs, k);
     const int tid = threadIdx.x;
-    for (int i = tid; i < S.len; i += kWG) acc[i] = 0.0f;
+    for (int i = tid; i < S.len; i += WG) acc[i] = 0.0f;
     __syncthreads();
 
-    if (S.kb <= kWG) {
+    if (S.kb <= WG) {
         // thread tid holds column tid of kBatchRows consecutive rows.  Requests are
         // unconditional (row and column clamped into the window) and their results stay as
         // loaded until they are applied, so that all of a batch is in flight at once.
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs,
         for (int r = 0; r < m_rows; ++r) {
             const float c = coef[r];
             const int64_t at = (int64_t)r * k + S.col0;
-            for (int j = tid; j < S.kb; j += kWG) {
+            for (int j = tid; j < S.kb; j += WG) {
                 const int ix = I[at + j];
                 const float term = c * widen(V[at + j]);
                 if ((unsigned)ix < (unsigned)S.len) acc[ix] = acc[ix] + term;
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kWG) void sparse_combine_kernel(int64_t d, int dbs,
     }
 
     TO *dst = out + S.e0;
-    for (int i = tid; i < S.len; i += kWG) narrow(dst + i, widen(dst[i]) + acc[i]);
+    for (int i = tid; i < S.len; i += WG) narrow(dst + i, widen(dst[i]) + acc[i]);
 }
 
 // ---- copy_values with typed window values ---------------------------------------------------
@@ -311,13 +311,18 @@ int ma_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d
     const int lds = (int)(d_block_size * 4);
     if (lds > kLdsBytes) return MA_ERR_LDS;
     hipStream_t s = (hipStream_t)stream;
-#define CALL(TO, TV)                                                                            \
-    if ((rc = allow_lds(sparse_combine_kernel<TO, TV>, lds))) return rc;                        \
-    sparse_combine_kernel<TO, TV><<<(unsigned)nblocks, kWG, lds, s>>>(                          \
+    // rows of at most 256 entries go to 256-thread workgroups: a row's barrier then joins four
+    // waves instead of eight
+#define CALL_WG(TO, TV, WG)                                                                     \
+    if ((rc = allow_lds(sparse_combine_kernel<TO, TV, WG>, lds))) return rc;                    \
+    sparse_combine_kernel<TO, TV, WG><<<(unsigned)nblocks, WG, lds, s>>>(                       \
         d, (int)d_block_size, (int)k_block_size, k, (int)m_rows, coef, indices,                 \
         (const TV *)values, (TO *)out);
+#define CALL(TO, TV)                                                                            \
+    if (k_block_size <= 256) { CALL_WG(TO, TV, 256) } else { CALL_WG(TO, TV, kWG) }
     MA_DISPATCH2(out_dtype, values_dtype, CALL)
 #undef CALL
+#undef CALL_WG
     return (int)hipGetLastError();
 }
 
