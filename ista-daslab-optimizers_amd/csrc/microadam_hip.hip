@@ -440,7 +440,9 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
 // which of them they fill and which they consume.
 //   FULL: the block has exactly kRound*C elements, so no chunk needs a bounds check.
 //   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
-template <class R, bool FULL, int QL>
+//   HOLD: the general window stage may keep the block's window entries in registers (40 of
+//         them), for kernels compiled with the register budget of two workgroups per CU.
+template <class R, bool FULL, int QL, bool HOLD = false>
 struct FusedBlock {
     typedef typename R::elem_t elem_t;
     static constexpr int C = R::kC;
@@ -461,6 +463,11 @@ struct FusedBlock {
     Divisor d15;
     PhaseTimer pt;
 
+    // window entries of the block, two per register as they lie in memory (index pairs in
+    // hI, value pairs in hV): step s = (row, trip) holds pair trip * kWG + tid of the row
+    static constexpr int kHold = HOLD ? 20 : 1;
+    uint32_t hI[kHold], hV[kHold];   //                      load_held          -> update
+    bool holding;
     RawChunk<R> praw[C];          // parameters              load_params_window -> update
     uint32_t entI[kEnt];          // entries of the older window rows, kept as loaded so that
     uint32_t entV[kEnt];          // nothing waits for them    load_params_window -> update
@@ -497,6 +504,7 @@ struct FusedBlock {
         d15.r = 0x1.111112p-4f;
         slot_clear = false;
         row_in_lds = true;
+        holding = false;
         pt.begin();
     }
 
@@ -531,6 +539,114 @@ struct FusedBlock {
                     const int64_t at = (int64_t)row * G.D.k + G.col0 + (e - row * G.kb);
                     entI[i] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
                     entV[i] = G.D.V[at];
+                }
+            }
+        }
+    }
+
+    // ---- the whole window of the block into registers, for the general window stage
+    // Entries travel two per 32-bit load, so every row of the block has to start on a 4-byte
+    // boundary and hold an even number of entries; otherwise, or when the window has more
+    // than kHold steps, the stage streams the entries as window_accumulate does.
+    __device__ __forceinline__ bool can_hold(const BlockGeo &G) const {
+        const int pairs = G.kb >> 1;
+        const int trips = (pairs + kWG - 1) / kWG;
+        return HOLD && P.L.cell_bytes == 0 && ((G.kb | G.D.k | G.col0) & 1) == 0 &&
+               (((uintptr_t)G.D.I | (uintptr_t)G.D.V) & 3) == 0 && P.W.rows * trips <= kHold;
+    }
+
+    // current == false: the older rows, from memory (can be asked for before the selection);
+    // current == true: the row this step selected, from LDS
+    __device__ __forceinline__ void load_held(const BlockGeo &G, bool current) {
+        if (!current) holding = can_hold(G);
+        if (!holding) return;
+        const int pairs = G.kb >> 1;
+        const int trips = (pairs + kWG - 1) / kWG;
+        const uint32_t *I2 = reinterpret_cast<const uint32_t *>(G.D.I + G.col0);
+        const uint32_t *V2 = reinterpret_cast<const uint32_t *>(G.D.V + G.col0);
+        const int64_t k2 = G.D.k >> 1;
+        int row = 0, it = 0;  // uniform
+#pragma unroll
+        for (int s = 0; s < kHold; ++s) {
+            if (!current) {
+                hI[s] = 0xffffffffu;  // index 0xffff lies in no range
+                hV[s] = 0;
+            }
+            if (row < P.W.rows) {
+                const int w = it * kWG + tid;
+                if (w < pairs) {
+                    const bool from_lds = row == G.D.row && row_in_lds;
+                    if (current && from_lds) {
+                        hI[s] = reinterpret_cast<const uint32_t *>(sel_idx)[w];
+                        hV[s] = reinterpret_cast<const uint32_t *>(sel_val)[w];
+                    } else if (!current && !from_lds) {
+                        hI[s] = I2[row * k2 + w];
+                        hV[s] = V2[row * k2 + w];
+                    }
+                }
+                if (++it == trips) {
+                    it = 0;
+                    ++row;
+                }
+            }
+        }
+    }
+
+    // window_accumulate from the held entries: same order of additions (rows in increasing
+    // order, a barrier after each row; the two entries of a register are distinct coordinates)
+    __device__ __forceinline__ void accumulate_held(int kb, int lo, int hi) {
+        for (int i = tid; i < hi - lo; i += kWG) {
+            z1[i] = 0.0f;
+            z2[i] = 0.0f;
+        }
+        __syncthreads();
+        pt.mark(12);
+        const int trips = ((kb >> 1) + kWG - 1) / kWG;
+        const uint32_t span = (uint32_t)(hi - lo);
+        // lane l keeps the weights of row l (a window has at most 64 rows), handed out by
+        // readlane: no memory access per step
+        const float w1v = P.W.w1[lane], w2v = P.W.w2[lane];
+        int row = 0, it = 0;  // uniform
+#pragma unroll
+        for (int s = 0; s < kHold; ++s) {
+            if (row < P.W.rows) {
+                const uint32_t c0 = (hI[s] & 0xffffu) - (uint32_t)lo, c1 = (hI[s] >> 16) - (uint32_t)lo;
+                // rows written by these kernels are in increasing coordinate order, so a range
+                // is a stretch of lanes: most waves have nothing to add and skip the rest
+                if (__builtin_amdgcn_ballot_w64(c0 < span || c1 < span) != 0) {
+                    const uint32_t b0 = hV[s] & 0xffffu, b1 = hV[s] >> 16;
+                    const bool ok0 = c0 < span && (b0 & 0x7fffu) != 0;
+                    const bool ok1 = c1 < span && (b1 & 0x7fffu) != 0;
+                    const float w1 =
+                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w1v), row));
+                    const float w2 =
+                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w2v), row));
+                    const float v0 = bf2f(b0), v1 = bf2f(b1);
+                    const float a10 = w1 * v0, a11 = w1 * v1;
+                    const float q0 = v0 * v0, q1 = v1 * v1;
+                    const float a20 = w2 * q0, a21 = w2 * q1;
+                    float r10 = 0.0f, r20 = 0.0f, r11 = 0.0f, r21 = 0.0f;
+                    if (ok0) {
+                        r10 = z1[c0];
+                        r20 = z2[c0];
+                    }
+                    if (ok1) {
+                        r11 = z1[c1];
+                        r21 = z2[c1];
+                    }
+                    if (ok0) {
+                        z1[c0] = r10 + a10;
+                        z2[c0] = r20 + a20;
+                    }
+                    if (ok1) {
+                        z1[c1] = r11 + a11;
+                        z2[c1] = r21 + a21;
+                    }
+                }
+                if (++it == trips) {
+                    it = 0;
+                    ++row;
+                    __syncthreads();
                 }
             }
         }
@@ -794,7 +910,11 @@ struct FusedBlock {
         __syncthreads();  // the LDS of the selection is reused below
         for (int lo = 0; lo < n; lo += P.L.sub_len) {
             const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
-            window_accumulate(wv, G.kb, lo, hi, z1, z2);
+            if (HOLD && holding)
+                accumulate_held(G.kb, lo, hi);
+            else
+                window_accumulate(wv, G.kb, lo, hi, z1, z2);
+            pt.mark(13);
             for (int c = tid; c < hi - lo; c += kWG) {
                 float u = 0.0f;
                 if (z1[c] != 0.0f || z2[c] != 0.0f)
@@ -802,6 +922,7 @@ struct FusedBlock {
                 z1[c] = R::kBF16 ? bf2f(f2bf(u)) : u;
             }
             __syncthreads();
+            pt.mark(14);
             // store addresses formed afresh, as in param_stage
             const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
 #pragma unroll
@@ -822,6 +943,7 @@ struct FusedBlock {
                 }
             }
             __syncthreads();
+            pt.mark(15);
         }
         pt.mark(16);
     }
@@ -1638,7 +1760,7 @@ __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
 
 // One workgroup per block: any block shape.  Tensor i contributes its blocks
 // blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
-template <class R, int MIN_WAVES, int QL, bool DENSE = false>
+template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int ti = find_tensor(P, (int)blockIdx.x);
@@ -1646,6 +1768,8 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     auto run = [&](auto &fb) {
         fb.load_grad_inputs(G);
         fb.dequant(G);
+        // the older window rows are most of this path's traffic: asked for before the selection
+        if constexpr (HOLD) fb.load_held(G, false);
         fb.topk_and_row(G);
         if constexpr (DENSE) {
             fb.quantize_dense(G);
@@ -1657,6 +1781,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
             // asked for only now: measured faster than at the start of the block, where they
             // keep 30 more registers live through the selection and the quantisation
             fb.load_params_window(G);
+            if constexpr (HOLD) fb.load_held(G, true);
             fb.update(G);
         }
     };
@@ -1665,14 +1790,14 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
 #else
     if (G.n == R::kC * kRound) {
 #endif
-        FusedBlock<R, true, QL> fb(P, lds);
+        FusedBlock<R, true, QL, HOLD> fb(P, lds);
         run(fb);
 #ifdef MA_ANALYZE_FULL_ONLY
     } else if (false) {
 #else
     } else {
 #endif
-        FusedBlock<R, false, QL> fb(P, lds);
+        FusedBlock<R, false, QL, HOLD> fb(P, lds);
         run(fb);
     }
 }
@@ -1848,14 +1973,16 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
     return MA_ERR_BLOCK_SIZE;
 }
 
-template <class R, int QL, bool DENSE = false>
+template <class R, int QL, bool DENSE = false, bool HOLD = false>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // bf16 blocks of up to 20480 elements fit 80 registers and a third of the LDS: three
-    // workgroups per CU
-    constexpr int kWaves_ = (R::kBF16 && R::kC <= kClass2) ? kWavesThreeWG : kMinWaves;
-    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE>, lds_bytes);
+    // workgroups per CU; the general window stage with the window held in registers takes the
+    // budget of two
+    constexpr int kWaves_ =
+        (R::kBF16 && R::kC <= kClass2 && !HOLD) ? kWavesThreeWG : kMinWaves;
+    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD>, lds_bytes);
     if (rc) return rc;
-    fused_step_kernel<R, kWaves_, QL, DENSE><<<grid, kWG, lds_bytes, s>>>(P);
+    fused_step_kernel<R, kWaves_, QL, DENSE, HOLD><<<grid, kWG, lds_bytes, s>>>(P);
     return launch_status();
 }
 
@@ -1879,6 +2006,13 @@ static int launch_fused_dense(int C, unsigned grid, int lds_bytes, hipStream_t s
 template <template <int> class RT>
 static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // the hardware-sized block gets kernels with the quantisation group size compiled in
+    if constexpr (RT<kClass2>::kBF16) {
+        // windows too large for the one-pass stage: the general stage, window in registers
+        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 6)
+            return launch_fused_one<RT<kClass2>, 8, false, true>(grid, lds_bytes, s, P);
+        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 5)
+            return launch_fused_one<RT<kClass2>, 4, false, true>(grid, lds_bytes, s, P);
+    }
     if (C == kClass2 && P.q_shift == 6) return launch_fused_one<RT<kClass2>, 8>(grid, lds_bytes, s, P);
     if (C == kClass2 && P.q_shift == 5) return launch_fused_one<RT<kClass2>, 4>(grid, lds_bytes, s, P);
     switch (C) {

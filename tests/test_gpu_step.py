@@ -64,6 +64,11 @@ CASES = [
     ([32768 + 1000], torch.bfloat16, 3, 128, 0.01, 0.0, 0.0, 32768, 5),
     ([10240 * 2 + 8], torch.bfloat16, 3, 8, 0.01, 0.0, 0.0, 10240, 5),
     ([1001, 777], torch.bfloat16, 3, 64, 0.03, 0.0, 0.0, 20480, 5),   # odd d: partial chunks
+    # windows too large for the one-pass stage (20 rows of 5 %): the general stage, with the
+    # window held in registers (even k), streamed (odd k; more rows than the registers hold)
+    ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.05, 0.0, 0.0, 20480, 23),
+    ([20480 * 2 + 4096, 20480], torch.bfloat16, 20, 64, 0.05, 0.0, 0.01, 20480, 22),
+    ([20480 + 8192], torch.bfloat16, 24, 32, 0.05, 0.0, 0.0, 20480, 26),
 ]
 
 
