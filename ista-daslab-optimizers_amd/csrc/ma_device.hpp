@@ -272,7 +272,10 @@ __device__ __forceinline__ void store8(uint16_t *base, int off, int n, bool vec,
         q.y = f2bf_pair(v[2], v[3]);
         q.z = f2bf_pair(v[4], v[5]);
         q.w = f2bf_pair(v[6], v[7]);
-        *reinterpret_cast<uint4 *>(base + off) = q;
+        // written once, not read again by this kernel: streamed past the caches
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u4 t = {q.x, q.y, q.z, q.w};
+        __builtin_nontemporal_store(t, reinterpret_cast<u4 *>(base + off));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i)
