@@ -29,6 +29,14 @@ CASES = {
     "f32_alpha_minus2": ([2000], "f32", 3, 64, 0.02, -2, 0.0, 1024, 4),
 }
 
+# Sparse M-FAC's window kernels (scalar products, linear combination) on the final window of
+# tensor 0 of a case above: name -> (case, live rows)
+SPARSE_CASES = {
+    "sparse_bf16_q64": ("bf16_q64", 4),
+    "sparse_bf16_block20480": ("bf16_block20480", 2),
+    "sparse_f32_q64_wd": ("f32_q64_wd", 3),
+}
+
 
 def main():
     out = {}
@@ -58,6 +66,25 @@ def main():
             out[f"{name}/min_vals/{i}"] = st["min_vals"].copy()
             out[f"{name}/max_vals/{i}"] = st["max_vals"].copy()
             out[f"{name}/index/{i}"] = np.int64(st["index"])
+    rng2 = np.random.default_rng(20240614)  # its own stream: the arrays above stay as they were
+    for name, (case, rows) in SPARSE_CASES.items():
+        sizes, dtype, m, q, k_init, alpha, wd, DB, steps = CASES[case]
+        d = sizes[0]
+        geo = oracle.geometry(d, DB, k_init, q)
+        I, V = out[f"{case}/I/0"], out[f"{case}/V/0"]
+        if dtype == "f32":  # fp32 vectors go with fp32 values (use_bf16 = False)
+            V = oracle.bf16_to_f32(V)
+        g = rng2.standard_normal(d).astype(np.float32)
+        g = oracle.f32_to_bf16(g) if dtype == "bf16" else g
+        coef = rng2.standard_normal(m).astype(np.float32)
+        dots = np.zeros(m)
+        oracle.sparse_scalar_products(d, rows, geo["k"], geo["d_block_size"],
+                                      geo["k_block_size_many"], g, I, V, dots)
+        comb = np.zeros(d, dtype=g.dtype)
+        oracle.sparse_linear_combination(d, rows, geo["k"], geo["d_block_size"],
+                                         geo["k_block_size_many"], coef, I, V, comb)
+        out[f"{name}/g"], out[f"{name}/coef"] = g, coef
+        out[f"{name}/dots"], out[f"{name}/comb"] = dots, comb
     np.savez_compressed(os.path.join(HERE, "microadam_small.npz"), **out)
     print("wrote", len(out), "arrays")
 

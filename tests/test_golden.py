@@ -58,3 +58,54 @@ def test_gpu_reproduces_fixture(oracle, name, use_fused):
         for key in KEYS:
             assert np.array_equal(got[key].reshape(-1), z[f"{name}/{key}/{i}"].reshape(-1)), key
         assert st["index"] == int(z[f"{name}/index/{i}"])
+
+
+# ---- Sparse M-FAC's window kernels on the final windows of the cases above --------------------
+
+from golden.make_golden import SPARSE_CASES  # noqa: E402
+
+
+def _sparse_inputs(oracle, z, name):
+    case, rows = SPARSE_CASES[name]
+    sizes, dtype, m, q, k_init, alpha, wd, DB, steps = CASES[case]
+    d = sizes[0]
+    geo = oracle.geometry(d, DB, k_init, q)
+    I, V = z[f"{case}/I/0"], z[f"{case}/V/0"]
+    if dtype == "f32":
+        V = oracle.bf16_to_f32(V)
+    return d, rows, m, geo["k"], geo["d_block_size"], geo["k_block_size_many"], I, V
+
+
+@pytest.mark.parametrize("name", sorted(SPARSE_CASES))
+def test_oracle_reproduces_sparse_fixture(oracle, name):
+    z = _load()
+    d, rows, m, k, dbs, kb, I, V = _sparse_inputs(oracle, z, name)
+    dots = np.zeros(m)
+    oracle.sparse_scalar_products(d, rows, k, dbs, kb, z[f"{name}/g"], I, V, dots)
+    assert np.array_equal(dots, z[f"{name}/dots"])
+    comb = np.zeros(d, dtype=z[f"{name}/g"].dtype)
+    oracle.sparse_linear_combination(d, rows, k, dbs, kb, z[f"{name}/coef"], I, V, comb)
+    assert np.array_equal(comb, z[f"{name}/comb"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(SPARSE_CASES))
+def test_gpu_reproduces_sparse_fixture(oracle, name):
+    """Linear combination bit for bit; scalar products within 2e-6 of the sum of the absolute
+    terms (the order of the device's fp32 sum is its own)."""
+    import torch
+    import ista_daslab_cuda_sparse_mfac as smf
+    from gpu_util import to_np, to_torch
+    z = _load()
+    d, rows, m, k, dbs, kb, I, V = _sparse_inputs(oracle, z, name)
+    g, Id, Vd = to_torch(z[f"{name}/g"]), torch.from_numpy(I.copy()).cuda(), to_torch(V)
+    bf16 = int(g.dtype == torch.bfloat16)
+    dots = torch.zeros(m, dtype=torch.float32, device="cuda")
+    smf.SP(0, 0, 23, d, rows, k, dbs, kb, g, Id, Vd, dots, bf16)
+    pos = (torch.arange(k) // kb) * dbs + torch.from_numpy(I.astype(np.int64))
+    mass = (Vd.cpu().double().abs() * g.cpu().double()[pos].abs()).sum(dim=1).numpy()
+    assert np.all(np.abs(dots.cpu().numpy() - z[f"{name}/dots"]) <= 2e-6 * mass + 1e-30)
+    comb = torch.zeros(d, dtype=g.dtype, device="cuda")
+    smf.LCG(0, 0, 51, d, rows, k, dbs, kb, torch.from_numpy(z[f"{name}/coef"]).cuda(), Id, Vd,
+            comb, bf16)
+    assert np.array_equal(to_np(comb), z[f"{name}/comb"])
