@@ -364,6 +364,9 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op))
                      if args.storage is None else None,
+                     # achieved and traffic are both per step (10 launches of the block kernel
+                     # at 7B): algorithmic bytes of a step / device time of a step
+                     "per": "step", "algorithmic_bytes": bpp * n_params,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},
     }
