@@ -55,7 +55,6 @@ __global__ __launch_bounds__(kWG) void sparse_dot_kernel(int64_t d, int dbs, int
     const BlockSpan S = block_span(d, dbs, kbs, k);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     TG *gl = (TG *)lds_raw;
-    float *rowsum = (float *)(lds_raw + (((size_t)dbs * sizeof(TG) + 15) & ~(size_t)15));
 
     const TG *src = g + S.e0;
     constexpr int kPer16 = 16 / sizeof(TG);
@@ -107,14 +106,14 @@ __global__ __launch_bounds__(kWG) void sparse_dot_kernel(int64_t d, int dbs, int
             accA += __shfl_xor(accA, s, 64);
             accB += __shfl_xor(accB, s, 64);
         }
+        // straight to the workspace: LDS holds the block of g and nothing else, so that four
+        // workgroups with a 20480-element bf16 block share a CU
         if (lane == 0) {
-            rowsum[r] = accA;
-            if (two) rowsum[r2] = accB;
+            float *dst = partial + (int64_t)blockIdx.x * m_rows;
+            dst[r] = accA;
+            if (two) dst[r2] = accB;
         }
     }
-    __syncthreads();
-    float *dst = partial + (int64_t)blockIdx.x * m_rows;
-    for (int r = row_lo + tid; r < row_hi; r += kWG) dst[r] = rowsum[r];
 }
 
 // out[r] += sum over blocks of partial[b][r]: a wave per row, lane l adds blocks l, l + 64, ...
@@ -277,7 +276,7 @@ int ma_sparse_scalar_products(int64_t d, int64_t m_rows, int64_t k, int64_t d_bl
         workspace_bytes < nblocks * m_rows * (int64_t)sizeof(float))
         return MA_ERR_ARG;
     const int esize = g_dtype == MA_F32 ? 4 : 2;
-    const int lds = (int)(((d_block_size * esize + 15) & ~(int64_t)15) + m_rows * 4);
+    const int lds = (int)((d_block_size * esize + 15) & ~(int64_t)15);
     if (lds > kLdsBytes) return MA_ERR_LDS;
     hipStream_t s = (hipStream_t)stream;
     float *partial = (float *)workspace;
