@@ -348,7 +348,10 @@ struct TensorDesc {
     int32_t blk0;         // block of the tensor that its first work item stands for
     float *ws;            // two-pass route: per-block extremes of the residual, else unused
 };
-constexpr int kTensorsPerLaunch = 24;
+// The descriptors travel by value in the kernel arguments (112 bytes each; the runtime passes
+// arguments of this size intact).  Fewer, longer launches: each launch ends with a partly
+// filled round of workgroups, and small tensors would otherwise queue up behind each other.
+constexpr int kTensorsPerLaunch = 112;
 
 struct FusedParams {
     TensorDesc t[kTensorsPerLaunch];
@@ -1755,10 +1758,13 @@ struct FusedBlock {
 
 // which tensor owns workgroup / work item `w` of the launch (first_block is ascending)
 __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
-    int ti = 0;
-    for (int i = 1; i < P.n_tensors; ++i)
-        if (w >= P.t[i].first_block) ti = i;
-    return ti;
+    // the last tensor whose first work item is not beyond w
+    int lo = 0, hi = P.n_tensors - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (w >= P.t[mid].first_block) lo = mid; else hi = mid - 1;
+    }
+    return lo;
 }
 
 // One workgroup per block: any block shape.  Tensor i contributes its blocks
