@@ -2403,6 +2403,12 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             dbs_max = kb_max = 0;
             return rc;
         };
+        // the class's tensors are spread evenly over as few launches as hold them
+        int in_class = 0;
+        for (int i = 0; i < n_tensors; ++i)
+            if (chunks_for(geometry(tensors[i].d, h->d_block_size, h->k_init).dbs) == C) ++in_class;
+        const int launches = (in_class + kTensorsPerLaunch - 1) / kTensorsPerLaunch;
+        const int per_launch = launches ? (in_class + launches - 1) / launches : 0;
         int64_t ws_off = 0;
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
@@ -2411,7 +2417,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             if (span) ws_off += span_ws_bytes(&t, h);
             if (chunks_for(g.dbs) != C) continue;
             const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
-            if (count == kTensorsPerLaunch || items + nb > 0x7fffffff) {
+            if (count == per_launch || items + nb > 0x7fffffff) {
                 const int rc = flush();
                 if (rc) return rc;
             }
