@@ -144,6 +144,7 @@ class MicroAdam(torch.optim.Optimizer):
         logging_step = self._logging_active() and self.steps % self.log_interval == 0
 
         fused, spanning, dense = [], [], []  # (p, st, lr, wd)
+        log_after = []  # tensors a fused kernel steps on a logging step: metrics taken afterwards
         for group in self.param_groups:
             lr = group['lr']
             wd = group.get('weight_decay', self.weight_decay)
@@ -161,8 +162,14 @@ class MicroAdam(torch.optim.Optimizer):
                     self._initialize_parameter_state(p, lr, wd)
                 self._repair_state(st)
 
-                route = self._fusable(p, st) if self.use_fused and not logging_step else 0
+                route = self._fusable(p, st) if self.use_fused else 0
+                if logging_step and not (route in (1, 2) and self.alpha == 0):
+                    # with alpha != 0 the update holds a term that no state keeps: op by op
+                    route = 0
                 if route:
+                    if logging_step:
+                        norm_g += p.grad.view(-1).norm(p=2) ** 2  # the spanning route overwrites g
+                        log_after.append((p, st))
                     (fused, spanning, dense)[route - 1].append((p, st, lr, wd))
                     continue
 
@@ -180,6 +187,11 @@ class MicroAdam(torch.optim.Optimizer):
             self._fused_step(spanning, spanning=True)
         if dense:
             self._fused_step(dense, dense=True)
+        for p, st in log_after:
+            nu, ne, sp_u = self._metrics_after_fused_step(p, st)
+            norm_u += nu
+            norm_e += ne
+            sparsity_u += sp_u
 
         time_end = time.time()
         elapsed_step = time_end - time_start
@@ -456,6 +468,27 @@ class MicroAdam(torch.optim.Optimizer):
             norm_e = grad.norm(p=2) ** 2
 
         return norm_qe, norm_g, norm_u, norm_e, sp_u, sp_qe
+
+    def _metrics_after_fused_step(self, p, st):
+        """norm_u, norm_e and the update's zero count (micro_adam.py:306-308, :320-324) for a
+        tensor that a fused kernel has just stepped with alpha == 0: the update is rebuilt from
+        the window (which already holds this step's row, as at micro_adam.py:277-291) and the
+        error norm from the stored error feedback, both in p.grad, which the step leaves as
+        scratch like the reference does (:276, :321)."""
+        grad = p.grad.view(-1)
+        d = st['d']
+        grad.zero_()
+        ista_daslab_cuda_micro_adam.compute_microadam_update(
+            st['blocks'], self.threads, self.shared_memory_carveout, self.steps, self.beta1,
+            self.beta2, self.eps, st['d_block_size'], st['k_block_size_many'], d, self.m, st['k'],
+            st['I'], st['V'], grad)
+        norm_u = grad.norm(p=2) ** 2
+        sp_u = (grad == 0).sum()
+        grad.zero_()
+        ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, st['error'],
+                                                          st['min_vals'], st['max_vals'], grad, 1.0)
+        norm_e = grad.norm(p=2) ** 2
+        return norm_u, norm_e, sp_u
 
     # ------------------------------------------------------------------ logging (micro_adam.py:330-350)
     @staticmethod

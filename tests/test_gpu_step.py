@@ -313,3 +313,42 @@ def test_window_rows_that_name_the_same_coordinates(oracle, use_fused):
     I = opt.state[gp]["I"][:, :205].long()
     common = sum(len(set(I[0].tolist()) & set(I[r].tolist())) for r in range(1, m)) / (205 * (m - 1))
     assert common > 0.8, common
+
+
+@pytest.mark.parametrize("q,sizes", [(64, [20480 * 2 + 4096, 768]), (24576, [20480 * 3 + 100])],
+                         ids=["fused", "spanning"])
+def test_logging_step_metrics_do_not_depend_on_the_route(q, sizes):
+    """On a logging step (micro_adam.py:155, :306-308, :320-324, :330-350) the fused routes take
+    their metrics after the kernel, from the window and the stored error feedback; the numbers
+    handed to _log must equal the op-by-op route's, and so must the state."""
+    from ista_daslab_optimizers import MicroAdam
+    logs = {}
+    opts = {}
+    for use_fused in (True, False):
+        gen = torch.Generator().manual_seed(11)
+        params = [torch.nn.Parameter((torch.randn(n, generator=gen) * 0.02).to(torch.bfloat16).cuda())
+                  for n in sizes]
+        opt = MicroAdam(params, m=4, lr=1e-3, quant_block_size=q, k_init=0.01, alpha=0,
+                        weight_decay=0.01)
+        opt.use_fused = use_fused
+        opt.log_interval = 2
+        opt._logging_active = lambda: True
+        seen = logs.setdefault(use_fused, [])
+        opt._log = lambda *a, seen=seen: seen.append([float(x) for x in a[:6]])
+        kernel_steps = []
+        inner = opt._fused_step
+        opt._fused_step = lambda *a, _o=opt, _i=inner, _k=kernel_steps, **kw: (_k.append(_o.steps),
+                                                                               _i(*a, **kw))
+        for s in range(6):
+            for p in params:
+                p.grad = (torch.randn(p.numel(), generator=gen) * 0.01).to(torch.bfloat16).cuda()
+            opt.step()
+        opts[use_fused] = (opt, params)
+        # the logging steps 2, 4, 6 went through the fused kernels too
+        assert sorted(set(kernel_steps)) == ([1, 2, 3, 4, 5, 6] if use_fused else [])
+    assert len(logs[True]) == 3 and logs[True] == logs[False], (logs[True], logs[False])
+    for pf, po in zip(opts[True][1], opts[False][1]):
+        assert torch.equal(pf.data, po.data)
+        sf, so = opts[True][0].state[pf], opts[False][0].state[po]
+        for key in ("error", "min_vals", "max_vals"):
+            assert torch.equal(sf[key], so[key]), key
