@@ -248,6 +248,72 @@ def bench_sparse_window(args):
     print(json.dumps(res))
 
 
+def calibration(args):
+    """Known-size streaming kernels on this device: the rate it sustains for reads, writes, a
+    copy, the step's 2:1 read:write mix and the step's three large streams, with the step's own
+    access shape (ma_stream_probe) and with stock torch kernels.  Prints one JSON line; the
+    same kernels are what the FETCH_SIZE / WRITE_SIZE counters are scaled against."""
+    import ctypes
+    import torch
+    from ista_daslab_optimizers import _hip
+    dev = torch.device("cuda:0")
+    nbytes = (args.calibration_gib << 30) // 40960 * 40960
+    a = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=dev).normal_()
+    b = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=dev).normal_()
+    c = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=dev)
+    e = torch.zeros(nbytes // 4, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    reps = max(3, args.steps)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(reps)]
+        for e0, e1 in ev:
+            e0.record()
+            fn()
+            e1.record()
+        torch.cuda.synchronize()
+        ms = sorted(x.elapsed_time(y) for x, y in ev)
+        return ms[len(ms) // 2]
+
+    def probe(mode, nt, wgs=0):
+        def run():
+            _hip.check(_hip.lib.ma_stream_probe(mode, nt, nbytes, wgs, a.data_ptr(), b.data_ptr(),
+                                                c.data_ptr(), e.data_ptr(), sink.data_ptr(),
+                                                _hip.stream_ptr()), "ma_stream_probe")
+        return run
+
+    moved = {0: nbytes, 1: nbytes, 2: 2 * nbytes, 3: 3 * nbytes, 4: 3 * nbytes + nbytes // 2}
+    names = {0: "read", 1: "write", 2: "copy", 3: "update (2 reads : 1 write)",
+             4: "step streams (g, p, EF read; p, EF written)"}
+    rows = []
+    for mode in range(5):
+        for nt in (1, 0):
+            for wgs in (0, 256 * 3 * 4):
+                ms = timed(probe(mode, nt, wgs))
+                rows.append({"kernel": "ma_stream_probe", "what": names[mode], "nontemporal": bool(nt),
+                             "workgroups": wgs or nbytes // 40960, "bytes": moved[mode], "ms": ms,
+                             "GB/s": moved[mode] / ms / 1e6})
+    rows.append({"kernel": "torch copy_", "what": names[2], "bytes": 2 * nbytes,
+                 "ms": (ms := timed(lambda: c.copy_(a))), "GB/s": 2 * nbytes / ms / 1e6})
+    rows.append({"kernel": "torch add(out=)", "what": "c = a + b (2 reads : 1 write)",
+                 "bytes": 3 * nbytes, "ms": (ms := timed(lambda: torch.add(a, b, out=c))),
+                 "GB/s": 3 * nbytes / ms / 1e6})
+    rows.append({"kernel": "torch add_", "what": names[3], "bytes": 3 * nbytes,
+                 "ms": (ms := timed(lambda: b.add_(a))), "GB/s": 3 * nbytes / ms / 1e6})
+    rows.append({"kernel": "torch fill_", "what": names[1], "bytes": nbytes,
+                 "ms": (ms := timed(lambda: c.fill_(1.0))), "GB/s": nbytes / ms / 1e6})
+    rows.append({"kernel": "torch sum", "what": names[0], "bytes": nbytes,
+                 "ms": (ms := timed(lambda: a.view(torch.int16).sum())),
+                 "GB/s": nbytes / ms / 1e6})
+    best = max(r["GB/s"] for r in rows if r["what"] == names[4])
+    print(json.dumps({"calibration": rows, "bytes_per_array": nbytes, "reps": reps,
+                      "peak_GB/s": HBM_PEAK_GBS, "step_streams_best_GB/s": best,
+                      "step_streams_best_frac_of_peak": best / HBM_PEAK_GBS}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -265,12 +331,17 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB -> 1 GiB device copy, as the known-size kernel "
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled against")
+    ap.add_argument("--calibration", action="store_true",
+                    help="time known-size streaming kernels instead of the optimizer step")
+    ap.add_argument("--calibration-gib", type=int, default=4, help="bytes per array, GiB")
     ap.add_argument("--storage", choices=["bf16", "f32"], default=None,
                     help="override the element type of parameters and gradients")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
 
+    if args.calibration:
+        return calibration(args)
     if args.workload == "sparse-mfac-resnet50":
         return bench_sparse_window(args)
 

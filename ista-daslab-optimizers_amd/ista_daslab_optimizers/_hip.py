@@ -71,6 +71,7 @@ def _load():
         "ma_sparse_linear_combination": (ci, [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp, ci,
                                               vp]),
         "ma_copy_values_typed": (ci, [i64, i64, i64, i64, vp, vp, vp, ci, ci, ci, vp]),
+        "ma_stream_probe": (ci, [ci, ci, i64, i64, vp, vp, vp, vp, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -86,7 +87,7 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified", "ma_spanning_step",
            "ma_spanning_step_workspace", "ma_spanning_step_check", "ma_sparse_scalar_products",
            "ma_sparse_scalar_products_workspace", "ma_sparse_linear_combination",
-           "ma_copy_values_typed")
+           "ma_copy_values_typed", "ma_stream_probe")
 
 
 def error_string(code):

@@ -147,12 +147,14 @@ def test_denormal_scale_gradients(oracle, scale, use_fused):
          grad_scale=scale)
 
 
-def test_config1_plumbing(oracle):
+@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
+def test_config1_plumbing(oracle, use_fused):
     """The plumbing configuration: one flat fp32 parameter, d = 1,048,576, N(0,1) gradients,
-    m=10, k=1 %, q=64, 20 steps, hardware block size."""
-    opt = _run(oracle, [1048576], torch.float32, 10, 64, 0.01, 0.0, 0.0, 20480, 20, True,
-               grad_scale=1.0, expect_route=True)
-    assert opt.d_block_size == 20480 and opt.steps == 20
+    m=10, k=1 %, q=64, hardware block size; run on to 100 steps (the configuration asks for 20;
+    the fp32 tolerance is stated after 100), state and parameters compared after every step."""
+    opt = _run(oracle, [1048576], torch.float32, 10, 64, 0.01, 0.0, 0.0, 20480, 100, use_fused,
+               grad_scale=1.0, expect_route=use_fused)
+    assert opt.d_block_size == 20480 and opt.steps == 100
 
 
 def test_outlier_gradients(oracle):
