@@ -38,9 +38,11 @@ extern "C" {
 #define MA_ERR_GEOMETRY (-4)    /* k / k_block_size inconsistent with d and d_block_size */
 #define MA_ERR_NOT_FUSABLE (-5) /* tensor does not meet ma_fused_step's layout conditions */
 #define MA_ERR_LDS (-6)         /* the launch would need more than 160 KB of LDS */
+#define MA_ERR_WORKSPACE (-7)   /* the list needs more than MA_STATIC_WORKSPACE_BYTES of scratch */
 
 #define MA_MAX_WINDOW 64 /* largest window length m the kernels take */
 #define MA_MAX_D_BLOCK 32768
+#define MA_STATIC_WORKSPACE_BYTES (8 << 20) /* scratch ma_spanning_step_static holds per GPU */
 #define MA_MAX_SPARSE_ROWS 4096 /* most window rows the Sparse M-FAC kernels take */
 
 const char *ma_error_string(int code);
@@ -199,6 +201,20 @@ int64_t ma_spanning_step_workspace(const ma_tensor *tensors /* host */, int n_te
 /* 0 if ma_spanning_step would accept this tensor, else the MA_ERR_* it would return. */
 int ma_spanning_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */,
                             double alpha);
+
+/* ma_spanning_step for callers that cannot allocate device memory or hand over a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments, conditions and results as ma_spanning_step;
+ * the per-block extremes of the residual go to a fixed array of MA_STATIC_WORKSPACE_BYTES
+ * (8 MiB) that the library holds in the memory of every GPU it runs on until the process ends,
+ * which is room for 524 288 top-k blocks per call (10.7e9 elements at d_block_size 20480); a
+ * list that needs more is rejected with MA_ERR_WORKSPACE and nothing is launched.  The call
+ * allocates and frees nothing.  The array's address is looked up at the first call on each
+ * device.  All calls on one GPU share that GPU's array: it need not be cleared between calls
+ * (the first pass writes every entry the second pass reads), but calls whose kernels may
+ * overlap on one GPU (different streams) race on it. */
+int ma_spanning_step_static(const ma_tensor *tensors /* host */, int n_tensors,
+                             const ma_hyper *hyper /* host */, double alpha, void *stream);
 
 /* ---- ista_daslab_cuda_sparse_mfac: the kernels that share the window layout -------------- */
 /* Sparse M-FAC (sparse_mfac/sparse_core_mfac_w_ef.py, SC below) keeps its m gradients in the

@@ -6,6 +6,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "../../include/microadam_hip.h"
 
 namespace ma {
@@ -2157,6 +2159,9 @@ const char *ma_error_string(int code) {
         case MA_ERR_GEOMETRY: return "k / k_block_size inconsistent with d and d_block_size";
         case MA_ERR_NOT_FUSABLE: return "tensor does not meet the fused step's layout conditions";
         case MA_ERR_LDS: return "launch would need more than 160 KB of LDS";
+        case MA_ERR_WORKSPACE:
+            return "list needs more workspace than ma_spanning_step_static holds "
+                   "(16 bytes per top-k block, MA_STATIC_WORKSPACE_BYTES in all)";
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "unknown error";
@@ -2478,6 +2483,49 @@ int64_t ma_spanning_step_workspace(const ma_tensor *tensors, int n_tensors, cons
 int ma_spanning_step(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, double alpha,
                       void *workspace, int64_t workspace_bytes, void *stream) {
     return step_impl(tensors, n_tensors, h, stream, true, alpha, workspace, workspace_bytes);
+}
+
+// ---- ma_spanning_step without a caller workspace and without any allocation -----------------
+// The per-block extremes of the residual go to a fixed array in device memory.  Every GPU the
+// library runs on holds its own copy of the array at its own address; the address is looked
+// up once per device, with that device current, and only that pointer is handed to kernels.
+constexpr int64_t kStaticScratchBytes = MA_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];  // per device, null until looked up
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return MA_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return MA_ERR_ARG;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+int ma_spanning_step_static(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
+                             double alpha, void *stream) {
+    if (!tensors || !h || n_tensors < 0) return MA_ERR_ARG;
+    int64_t need = 0;
+    for (int i = 0; i < n_tensors; ++i) {
+        if (tensors[i].d <= 0 || h->d_block_size < 1) return MA_ERR_ARG;
+        need += span_ws_bytes(&tensors[i], h);
+    }
+    if (need > kStaticScratchBytes) return MA_ERR_WORKSPACE;
+    void *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+    return step_impl(tensors, n_tensors, h, stream, true, alpha, ws, kStaticScratchBytes);
 }
 
 }  // extern "C"

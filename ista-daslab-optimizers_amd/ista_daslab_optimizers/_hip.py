@@ -13,6 +13,8 @@ LIB_PATH = os.path.join(_HERE, "libmicroadam_hip.so")
 MA_F32, MA_BF16 = 0, 1
 MA_ERR_NOT_FUSABLE = -5
 MA_ERR_LDS = -6
+MA_ERR_WORKSPACE = -7
+MA_STATIC_WORKSPACE_BYTES = 8 << 20
 MA_MAX_WINDOW = 64
 
 
@@ -60,6 +62,8 @@ def _load():
                                          ctypes.c_double, vp]),
         "ma_spanning_step": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
                                    ctypes.c_double, vp, ctypes.c_int64, vp]),
+        "ma_spanning_step_static": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
+                                          ctypes.c_double, vp]),
         "ma_spanning_step_workspace": (ctypes.c_int64, [ctypes.POINTER(MaTensor), ci,
                                                          ctypes.POINTER(MaHyper)]),
         "ma_spanning_step_check": (ci, [ctypes.POINTER(MaTensor), ctypes.POINTER(MaHyper),
@@ -85,7 +89,7 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_zerorize_block_components", "ma_asymm_block_quant", "ma_asymm_block_quant_inv",
            "ma_compute_microadam_update", "ma_block_topk", "ma_block_minmax", "ma_param_update",
            "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified", "ma_spanning_step",
-           "ma_spanning_step_workspace", "ma_spanning_step_check", "ma_sparse_scalar_products",
+           "ma_spanning_step_static", "ma_spanning_step_workspace", "ma_spanning_step_check", "ma_sparse_scalar_products",
            "ma_sparse_scalar_products_workspace", "ma_sparse_linear_combination",
            "ma_copy_values_typed", "ma_stream_probe")
 
