@@ -1,0 +1,10 @@
+// The fused step kernels for fp32 parameters and gradients (alpha == 0).
+#include "ma_block.hpp"
+
+namespace ma {
+
+int launch_fused_f32(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    return launch_fused<RegsF32>(C, grid, lds_bytes, s, P);
+}
+
+}  // namespace ma

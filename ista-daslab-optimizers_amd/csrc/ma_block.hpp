@@ -1,0 +1,1921 @@
+// The block kernels of the MicroAdam step: one 512-thread workgroup per top-k block, the block
+// held in registers.  Shared by the translation units that instantiate them (one per data type
+// and route, so that they compile side by side); gfx950 only.
+#pragma once
+#include "ma_device.hpp"
+
+#include "../../include/microadam_hip.h"
+
+namespace ma {
+
+
+// LDS map shared by the block kernels (byte offsets from the start of dynamic LDS)
+struct LdsMap {
+    int off_sel_idx;  // uint16[kb_max]
+    int off_sel_val;  // uint16[kb_max]
+    int off_slot;     // slot_cells cells of cell_bytes
+    int off_union;    // histograms and candidate lists during selection, then the window stage's arrays
+    int slot_cells;   // multiple of 8, >= longest block
+    int z_cap;        // entries the window stage's arrays hold
+    int sub_len;      // coordinates handled per window pass
+    int fast_cap;     // entries the one-pass window stage has room for, 0: none
+    int hist_log2;    // log2 of the histogram copies the general selection has room for
+    int compact;      // bf16 one-pass window stage with slots per coordinate instead of lists
+    int cell_bytes;   // width of a slot cell: 2, or 4 for fp32 data in the general window stage;
+                      // 0: no cells, the general window stage updates the parameters range by range
+    int total;        // bytes
+};
+constexpr int kMiscBytes = 256;  // the kSh* words at the very start
+constexpr int kFastTopkBytes = (2 * kSmallHistWords + 512) * 4;
+constexpr int kHistBytes =
+    257 * kHistCopies * 4 > kFastTopkBytes ? 257 * kHistCopies * 4 : kFastTopkBytes;
+
+struct WindowWeights {
+    float w1[kMaxWindow];
+    float w2[kMaxWindow];
+    float s1, s2, eps;
+    int rows;        // live rows: min(t, m)
+    int rows_total;  // m
+};
+
+// ---- the fused step -----------------------------------------------------------------------------------
+
+struct TensorDesc {
+    void *p;
+    const void *g;
+    uint8_t *err;
+    uint16_t *mn;
+    uint16_t *mx;
+    int16_t *I;
+    uint16_t *V;
+    int64_t d;
+    int64_t k;
+    int32_t row;
+    int32_t k_many;
+    int32_t k_few;
+    int32_t first_block;  // first work item of this tensor inside the launch
+    float neg_lr;
+    float decay;
+    int32_t apply_decay;
+    int32_t blk0;         // block of the tensor that its first work item stands for
+    float *ws;            // two-pass route: per-block extremes of the residual, else unused
+};
+// The descriptors travel by value in the kernel arguments (112 bytes each; the runtime passes
+// arguments of this size intact).  Fewer, longer launches: each launch ends with a partly
+// filled round of workgroups, and small tensors would otherwise queue up behind each other.
+constexpr int kTensorsPerLaunch = 112;
+
+struct FusedParams {
+    TensorDesc t[kTensorsPerLaunch];
+    WindowWeights W;
+    LdsMap L;
+    int32_t n_tensors;
+    int32_t d_block_size;
+    int32_t q_shift;  // log2(quant_block_size)
+    int32_t total_items;  // work items (blocks) of the launch
+    // two-pass route (quantisation blocks at least as long as the top-k blocks)
+    int32_t q_span;   // quantisation block length, a multiple of 8
+    float alpha;      // share of the dequantised error feedback added to the update
+    float keep;       // (float)(1 - alpha): share that stays in the error feedback
+};
+
+template <class R>
+struct RawChunk;
+template <int C>
+struct RawChunk<RegsBF16<C>> {
+    uint4 q;
+    __device__ __forceinline__ void load(const uint16_t *base, int off, int n, bool full) {
+        if (full || off + kChunk <= n) {
+            // read once: streamed past the caches (1 % on the 7B step)
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            const u4 t = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(base + off));
+            q = make_uint4(t.x, t.y, t.z, t.w);
+        } else {
+            uint32_t r[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (off + i < n) r[i >> 1] |= (uint32_t)base[off + i] << (16 * (i & 1));
+            q = make_uint4(r[0], r[1], r[2], r[3]);
+        }
+    }
+    __device__ __forceinline__ void to_float(float (&v)[8]) const {
+        const uint32_t r[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(r[i] << 16);
+            v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+        }
+    }
+};
+template <int C>
+struct RawChunk<RegsF32<C>> {
+    float v_[8];
+    __device__ __forceinline__ void load(const float *base, int off, int n, bool full) {
+        if (full) {
+            const float4 a = *reinterpret_cast<const float4 *>(base + off);
+            const float4 b = *reinterpret_cast<const float4 *>(base + off + 4);
+            v_[0] = a.x; v_[1] = a.y; v_[2] = a.z; v_[3] = a.w;
+            v_[4] = b.x; v_[5] = b.y; v_[6] = b.z; v_[7] = b.w;
+        } else {
+            load8(base, off, n, true, v_);
+        }
+    }
+    __device__ __forceinline__ void to_float(float (&v)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = v_[i];
+    }
+};
+
+// One-pass window stage: the rows * kb entries of a block are dealt out over the workgroup,
+// entry e to thread e % kWG, and requested at the start of the block.
+constexpr int kEnt = 5;        // entries per thread at most
+constexpr int kFastRows = 16;  // window rows at most: a coordinate's rows are a 16-bit mask
+
+// Where one top-k block lives: everything a stage needs to address it, copied out of the
+// launch parameters.  Wave-uniform (lives in scalar registers).
+struct BlockGeo {
+    TensorDesc D;
+    int64_t e0;    // first element
+    int64_t col0;  // first window column
+    int n;         // elements in the block
+    int kb;        // entries selected from it
+};
+
+__device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64_t b) {
+    BlockGeo G;
+    G.D = P.t[ti];
+    const int64_t d = G.D.d;
+    const int dbs = (int)(d < P.d_block_size ? d : P.d_block_size);
+    const int64_t n_full = d / dbs;
+    G.e0 = b * dbs;
+    G.n = (int)((d - G.e0) < dbs ? (d - G.e0) : dbs);
+    G.kb = b < n_full ? G.D.k_many : G.D.k_few;
+    G.col0 = b * G.D.k_many;
+    return G;
+}
+
+// The step of one block, cut into stages.  The register arrays are members; the stages say
+// which of them they fill and which they consume.
+//   FULL: the block has exactly kRound*C elements, so no chunk needs a bounds check.
+//   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
+//   HOLD: the general window stage may keep the block's window entries in registers (40 of
+//         them), for kernels compiled with the register budget of two workgroups per CU.
+template <class R, bool FULL, int QL, bool HOLD = false>
+struct FusedBlock {
+    typedef typename R::elem_t elem_t;
+    static constexpr int C = R::kC;
+
+    const FusedParams &P;
+    uint32_t *sh, *counter, *hist;
+    uint16_t *sel_idx, *sel_val, *coord;
+    // One LDS cell per coordinate of the block.  16 bits wide for bf16 data (window bookkeeping,
+    // then the update's bf16 bits) and in the one-pass window stage for fp32 data (bookkeeping,
+    // then 1 + the record that holds the update); 32 bits (the update's bits) for fp32 data in
+    // the general window stage.
+    uint16_t *cell16;
+    uint32_t *cell32;
+    float *z1, *z2;
+    int tid, lane, wave, q_shift, ql;
+    bool slot_clear;  // the slot cells are already zero when the update stage begins
+    bool row_in_lds;  // the window row of this step is taken from sel_idx / sel_val, not from HBM
+    Divisor d15;
+
+    // window entries of the block, two per register as they lie in memory (index pairs in
+    // hI, value pairs in hV): step s = (row, trip) holds pair trip * kWG + tid of the row
+    static constexpr int kHold = HOLD ? 20 : 1;
+    uint32_t hI[kHold], hV[kHold];   //                      load_held          -> update
+    bool holding;
+    RawChunk<R> praw[C];          // parameters              load_params_window -> update
+    uint32_t entI[kEnt];          // entries of the older window rows, kept as loaded so that
+    uint32_t entV[kEnt];          // nothing waits for them    load_params_window -> update
+    RawChunk<R> graw[C];          // gradient                load_grad_inputs   -> dequant
+    // 4-bit codes and statistics                            load_grad_inputs   -> dequant
+    // With a full block and a compile-time quantisation group the wave's statistics are
+    // fetched once, 64 per register (kCoStats registers per array), and handed to the lanes
+    // by cross-lane reads in dequant; otherwise every chunk loads its own pair.
+    static constexpr bool kCoop = FULL && QL > 0;
+    static constexpr int kWaveStats = kCoop ? C * kWave / (QL > 0 ? QL : 1) : 0;
+    static constexpr int kCoStats = kCoop ? (kWaveStats + kWave - 1) / kWave : 1;
+    uint32_t cw[C], smn[kCoop ? kCoStats : C], smx[kCoop ? kCoStats : C];
+    R r;                          // accumulator             dequant            -> quantize
+
+    __device__ __forceinline__ FusedBlock(const FusedParams &P_, unsigned char *lds) : P(P_) {
+        sh = reinterpret_cast<uint32_t *>(lds);
+        counter = sh + kShCounter;
+        sel_idx = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_idx);
+        sel_val = reinterpret_cast<uint16_t *>(lds + P.L.off_sel_val);
+        cell16 = reinterpret_cast<uint16_t *>(lds + P.L.off_slot);
+        cell32 = reinterpret_cast<uint32_t *>(lds + P.L.off_slot);
+        hist = reinterpret_cast<uint32_t *>(lds + P.L.off_union);
+        // without cells the sums of a coordinate range take everything from the cells' place on
+        z1 = reinterpret_cast<float *>(lds + (P.L.cell_bytes == 0 ? P.L.off_slot : P.L.off_union));
+        z2 = z1 + P.L.z_cap;
+        coord = reinterpret_cast<uint16_t *>(z2 + P.L.z_cap);
+        tid = threadIdx.x;
+        lane = tid & 63;
+        wave = tid >> 6;
+        q_shift = QL > 0 ? (QL == 4 ? 5 : 6) : P.q_shift;
+        ql = 1 << (q_shift - 3);
+        // 1/15 rounded to nearest; div_shared is exact for a reciprocal within one ulp
+        d15.u = 15.0f;
+        d15.r = 0x1.111112p-4f;
+        slot_clear = false;
+        row_in_lds = true;
+        holding = false;
+        wide = false;
+    }
+
+    __device__ __forceinline__ bool fast_window(const BlockGeo &G) const {
+        return P.W.rows * G.kb <= P.L.fast_cap && P.W.rows <= kFastRows && P.L.sub_len >= G.n;
+    }
+
+    // ---- parameters and the older window rows: requested early, consumed last
+    __device__ __forceinline__ void load_params_window(const BlockGeo &G) {
+        load_params(G);
+        wide = wide_window(G);
+        if (wide)
+            load_window_wide(G);
+        else
+            load_window(G);
+    }
+
+    __device__ __forceinline__ void load_params(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *p = reinterpret_cast<const elem_t *>(G.D.p) + G.e0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) praw[c].load(p, chunk_off<C>(wave, c, lane), n, FULL);
+    }
+
+    __device__ __forceinline__ void load_window(const BlockGeo &G) {
+        const bool fw = fast_window(G);
+        const int entries = fw ? P.W.rows * G.kb : 0;
+        const float rkb = __builtin_amdgcn_rcpf((float)G.kb);
+#pragma unroll
+        for (int i = 0; i < kEnt; ++i) {
+            entI[i] = entV[i] = 0;
+            if (__builtin_amdgcn_readfirstlane(wave) * kWave + i * kWG < entries) {
+                const int e = tid + i * kWG;
+                const int row = entry_row(e, rkb);
+                if (e < entries && (row != G.D.row || !row_in_lds)) {
+                    const int64_t at = (int64_t)row * G.D.k + G.col0 + (e - row * G.kb);
+                    entI[i] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
+                    entV[i] = G.D.V[at];
+                }
+            }
+        }
+    }
+
+    // ---- the whole window of the block into registers, for the general window stage
+    // Entries travel two per 32-bit load, so every row of the block has to start on a 4-byte
+    // boundary and hold an even number of entries; otherwise, or when the window has more
+    // than kHold steps, the stage streams the entries as window_accumulate does.
+    __device__ __forceinline__ bool can_hold(const BlockGeo &G) const {
+        const int pairs = G.kb >> 1;
+        const int trips = (pairs + kWG - 1) / kWG;
+        return HOLD && P.L.cell_bytes == 0 && ((G.kb | G.D.k | G.col0) & 1) == 0 &&
+               (((uintptr_t)G.D.I | (uintptr_t)G.D.V) & 3) == 0 && P.W.rows * trips <= kHold;
+    }
+
+    // current == false: the older rows, from memory (can be asked for before the selection);
+    // current == true: the row this step selected, from LDS
+    __device__ __forceinline__ void load_held(const BlockGeo &G, bool current) {
+        if (!current) holding = can_hold(G);
+        if (!holding) return;
+        const int pairs = G.kb >> 1;
+        const int trips = (pairs + kWG - 1) / kWG;
+        const uint32_t *I2 = reinterpret_cast<const uint32_t *>(G.D.I + G.col0);
+        const uint32_t *V2 = reinterpret_cast<const uint32_t *>(G.D.V + G.col0);
+        const int64_t k2 = G.D.k >> 1;
+        int row = 0, it = 0;  // uniform
+#pragma unroll
+        for (int s = 0; s < kHold; ++s) {
+            if (!current) {
+                hI[s] = 0xffffffffu;  // index 0xffff lies in no range
+                hV[s] = 0;
+            }
+            if (row < P.W.rows) {
+                const int w = it * kWG + tid;
+                if (w < pairs) {
+                    const bool from_lds = row == G.D.row && row_in_lds;
+                    if (current && from_lds) {
+                        hI[s] = reinterpret_cast<const uint32_t *>(sel_idx)[w];
+                        hV[s] = reinterpret_cast<const uint32_t *>(sel_val)[w];
+                    } else if (!current && !from_lds) {
+                        hI[s] = I2[row * k2 + w];
+                        hV[s] = V2[row * k2 + w];
+                    }
+                }
+                if (++it == trips) {
+                    it = 0;
+                    ++row;
+                }
+            }
+        }
+    }
+
+    // window_accumulate from the held entries: same order of additions (rows in increasing
+    // order, a barrier after each row; the two entries of a register are distinct coordinates)
+    __device__ __forceinline__ void accumulate_held(int kb, int lo, int hi) {
+        for (int i = tid; i < hi - lo; i += kWG) {
+            z1[i] = 0.0f;
+            z2[i] = 0.0f;
+        }
+        __syncthreads();
+        const int trips = ((kb >> 1) + kWG - 1) / kWG;
+        const uint32_t span = (uint32_t)(hi - lo);
+        // lane l keeps the weights of row l (a window has at most 64 rows), handed out by
+        // readlane: no memory access per step
+        const float w1v = P.W.w1[lane], w2v = P.W.w2[lane];
+        int row = 0, it = 0;  // uniform
+#pragma unroll
+        for (int s = 0; s < kHold; ++s) {
+            if (row < P.W.rows) {
+                const uint32_t c0 = (hI[s] & 0xffffu) - (uint32_t)lo, c1 = (hI[s] >> 16) - (uint32_t)lo;
+                // rows written by these kernels are in increasing coordinate order, so a range
+                // is a stretch of lanes: most waves have nothing to add and skip the rest
+                if (__builtin_amdgcn_ballot_w64(c0 < span || c1 < span) != 0) {
+                    const uint32_t b0 = hV[s] & 0xffffu, b1 = hV[s] >> 16;
+                    const bool ok0 = c0 < span && (b0 & 0x7fffu) != 0;
+                    const bool ok1 = c1 < span && (b1 & 0x7fffu) != 0;
+                    const float w1 =
+                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w1v), row));
+                    const float w2 =
+                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w2v), row));
+                    const float v0 = bf2f(b0), v1 = bf2f(b1);
+                    const float a10 = w1 * v0, a11 = w1 * v1;
+                    const float q0 = v0 * v0, q1 = v1 * v1;
+                    const float a20 = w2 * q0, a21 = w2 * q1;
+                    float r10 = 0.0f, r20 = 0.0f, r11 = 0.0f, r21 = 0.0f;
+                    if (ok0) {
+                        r10 = z1[c0];
+                        r20 = z2[c0];
+                    }
+                    if (ok1) {
+                        r11 = z1[c1];
+                        r21 = z2[c1];
+                    }
+                    if (ok0) {
+                        z1[c0] = r10 + a10;
+                        z2[c0] = r20 + a20;
+                    }
+                    if (ok1) {
+                        z1[c1] = r11 + a11;
+                        z2[c1] = r21 + a21;
+                    }
+                }
+                if (++it == trips) {
+                    it = 0;
+                    ++row;
+                    __syncthreads();
+                }
+            }
+        }
+    }
+
+    // row of window entry e when a row has 1 / rkb entries: (e + 0.5) / kb is at least 0.5 / kb
+    // away from an integer, far more than the rounding of the two operations
+    static __device__ __forceinline__ int entry_row(int e, float rkb) {
+        return (int)(((float)e + 0.5f) * rkb);
+    }
+
+    // ---- gradient, 4-bit error feedback and its statistics
+    __device__ __forceinline__ void load_grad_inputs(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+        const uint8_t *err = G.D.err + (G.e0 >> 1);
+        const uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        const uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            graw[c].load(g, off, n, FULL);
+            cw[c] = 0;
+            if constexpr (kCoop) {
+                cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
+                continue;
+            } else {
+                smn[c] = smx[c] = 0;
+            }
+            if (FULL || off < n) {
+                if (FULL || off + kChunk <= n) {
+                    cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        cw[c] |= (uint32_t)err[(off >> 1) + j] << (8 * j);
+                }
+                const unsigned qb = (unsigned)off >> q_shift;
+                smn[c] = mnp[qb];
+                smx[c] = mxp[qb];
+            }
+        }
+        if constexpr (kCoop) {
+            const unsigned wave_first = (unsigned)(wave * C * kWave) / (unsigned)QL;
+#pragma unroll
+            for (int i = 0; i < kCoStats; ++i) {
+                const unsigned j = (unsigned)(i * kWave + lane);
+                smn[i] = smx[i] = 0;
+                if (j < (unsigned)kWaveStats) {
+                    smn[i] = mnp[wave_first + j];
+                    smx[i] = mxp[wave_first + j];
+                }
+            }
+        }
+    }
+
+    // ---- a = g + Qinv(e), rounded to the element type (MA:190)
+    __device__ __forceinline__ void dequant(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float v[8];
+            graw[c].to_float(v);
+            uint32_t mnb, mxb;
+            if constexpr (kCoop) {
+                const int j0 = c * (kWave / QL);  // first statistic of this chunk in the wave
+                const int src = (j0 & (kWave - 1)) + lane / QL;
+                mnb = (uint32_t)__shfl((int)smn[j0 >> 6], src, kWave);
+                mxb = (uint32_t)__shfl((int)smx[j0 >> 6], src, kWave);
+            } else {
+                mnb = smn[c];
+                mxb = smx[c];
+            }
+            const float mn = bf2f(mnb), mx = bf2f(mxb);
+            const float u = div15(mx - mn, d15);
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                float deq = (float)code * u;
+                deq = deq + mn;
+                v[e] = v[e] + deq;
+            }
+            if (!FULL && off + kChunk > n) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (off + e >= n) v[e] = 0.0f;
+            }
+            r.set_chunk(c, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        launder(r);
+    }
+
+    // ---- block top-k (MA:193-200), gather (MA:202-209), zero (MA:214), window row write
+    __device__ __forceinline__ void topk_and_row(const BlockGeo &G) {
+        const int kb = G.kb;
+        bool topk_done = false;
+        if constexpr (FULL && R::kBF16) {
+            if (kb <= kWG) {
+                topk_done = fast_topk_bf16(r, kb, cell16, hist, sh, sel_idx, sel_val);
+                launder(r);
+                // the block was parked in the slot cells and every thread cleared its own
+                slot_clear = topk_done && P.L.slot_cells == C * kRound;
+            }
+        }
+        if (!topk_done) {
+            uint32_t T;
+            int take_eq;
+            select_threshold(r, kb, hist, sh, T, take_eq, P.L.hist_log2);
+            launder(r);
+            compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
+            launder(r);
+        }
+        int16_t *Irow = G.D.I + ((int64_t)G.D.row * G.D.k + G.col0);
+        uint16_t *Vrow = G.D.V + ((int64_t)G.D.row * G.D.k + G.col0);
+        for (int j = tid; j < kb; j += kWG) {
+            Irow[(unsigned)j] = (int16_t)sel_idx[j];
+            Vrow[(unsigned)j] = sel_val[j];
+        }
+    }
+
+    // ---- residual statistics (MA:217-228) and 4-bit codes (MA:231)
+    __device__ __forceinline__ void quantize(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        uint8_t *err = G.D.err + (G.e0 >> 1);
+        uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float x[8];
+            float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                x[e] = r.val(c, e);
+                if (FULL || off + e < n) {
+                    mn = fmin_raw(mn, x[e]);
+                    mx = fmax_raw(mx, x[e]);
+                }
+            }
+            group_minmax<QL>(mn, mx, ql);
+            const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
+            if (FULL || off < n) {
+                if ((lane & (ql - 1)) == 0) {
+                    const unsigned qb = (unsigned)off >> q_shift;
+                    mnp[qb] = (uint16_t)mnb;
+                    mxp[qb] = (uint16_t)mxb;
+                }
+                const float mnf = bf2f(mnb), mxf = bf2f(mxb);
+                const float u = div15(mxf - mnf, d15);
+                float cf[8];
+                codes8(x, mnf, u, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- Adam direction from the window (MA:277-291), then p = p * (1 - lr*wd) (MA:234-235)
+    //      and p += -lr * u (MA:304).  The slot cells end up holding the update's bits, 0
+    //      where no window row names the coordinate.
+    __device__ __forceinline__ void update(const BlockGeo &G) {
+        if (P.L.cell_bytes == 0) {
+            update_by_ranges(G);
+        } else if (wide) {
+            update_wide(G);
+        } else {
+            window_stage(G);
+            param_stage(G);
+        }
+    }
+
+    // =========================================================================================
+    // Window and parameter stage of a full bf16 block whose window fits one pass (the usual
+    // case: m = 10 rows of 1 %).  Against window_stage + param_stage:
+    //  * the older rows are fetched four entries per 8-byte load: thread t takes the entries
+    //    4w - a .. 4w - a + 3 of older row t / W (w = t % W, W loads per row, a = 1 if the
+    //    block's stretch of that row starts on an odd entry, so that every load is 4-byte
+    //    aligned), and entry t of the row this step selected, which is still in LDS;
+    //  * coordinates named by several rows are summed through lists: the entry of the lowest
+    //    row reserves one cell per row of the coordinate, every entry files its two terms at
+    //    its row's rank, the owner adds them in that order (the order of the rows, as in
+    //    compute_microadam_update): four barriers, no loop over rows;
+    //  * without weight decay only the coordinates the window names change, so the
+    //    parameters are parked in the coordinate cells, the owners of the updates change
+    //    their cells, and the block goes back to memory as it lies there: a few dozen
+    //    vector instructions instead of four per element.
+    // =========================================================================================
+    bool wide;                  // this block takes the stage below
+    uint32_t wI[2], wV[2];      // four entries of an older row: indices, values (bf16 bits)
+    int w_first, w_row;         // number of the first of the four in the block's stretch of
+                                // the row (-1 .. kb-1); the row, -1: none
+
+    __device__ __forceinline__ bool wide_window(const BlockGeo &G) const {
+        if constexpr (!(R::kBF16 && FULL)) {
+            return false;
+        } else {
+            if (!P.L.compact || !row_in_lds || !fast_window(G)) return false;
+            if ((((uintptr_t)G.D.I | (uintptr_t)G.D.V) & 3) != 0) return false;
+            const int W = G.kb / 4 + 1;
+            return older_rows(G) * W <= kWG && G.kb <= kWG && P.W.rows <= 15;
+        }
+    }
+
+    // live rows that come from memory: all but the row this step writes (which is live unless
+    // the caller's ring position and step count disagree; it is then written and not read)
+    __device__ __forceinline__ int older_rows(const BlockGeo &G) const {
+        return P.W.rows - (G.D.row < P.W.rows ? 1 : 0);
+    }
+
+    __device__ __forceinline__ void load_window_wide(const BlockGeo &G) {
+        struct __attribute__((aligned(4))) Pair32 {
+            uint32_t x, y;
+        };
+        const int W = G.kb / 4 + 1;
+        const int older = older_rows(G);
+        const int ro = (int)(((float)tid + 0.5f) * __builtin_amdgcn_rcpf((float)W));
+        const int w = tid - ro * W;
+        w_row = -1;
+        w_first = 0;
+        wI[0] = wI[1] = wV[0] = wV[1] = 0;
+        if (ro < older) {
+            const int row = (ro < G.D.row || G.D.row >= P.W.rows) ? ro : ro + 1;
+            const int64_t e_first = (int64_t)row * G.D.k + G.col0;
+            const int a = (int)(e_first & 1);
+            const int64_t e_base = e_first - a + 4 * w;
+            w_first = 4 * w - a;
+            w_row = row;
+            const uint16_t *Ip = reinterpret_cast<const uint16_t *>(G.D.I) + e_base;
+            const uint16_t *Vp = G.D.V + e_base;
+            if (e_base + 4 <= (int64_t)P.W.rows_total * G.D.k) {
+                const Pair32 qi = *reinterpret_cast<const Pair32 *>(Ip);
+                const Pair32 qv = *reinterpret_cast<const Pair32 *>(Vp);
+                wI[0] = qi.x; wI[1] = qi.y; wV[0] = qv.x; wV[1] = qv.y;
+            } else {  // the last load of the last row may not reach past the arrays
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (e_base + j < (int64_t)P.W.rows_total * G.D.k) {
+                        wI[j >> 1] |= (uint32_t)Ip[j] << (16 * (j & 1));
+                        wV[j >> 1] |= (uint32_t)Vp[j] << (16 * (j & 1));
+                    }
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void update_wide(const BlockGeo &G) {
+        if constexpr (R::kBF16 && FULL) update_wide_bf16(G);
+    }
+
+    __device__ __forceinline__ void update_wide_bf16(const BlockGeo &G) {
+        constexpr int n = C * kRound;
+        constexpr int kSlots = 5;  // four entries of an older row, one of this step's row
+        const TensorDesc &D = G.D;
+        const int kb = G.kb;
+        uint32_t *lcount = sh + kShLinks;
+        const int cap = (P.L.total - P.L.off_union) / 8;
+        float *f1 = reinterpret_cast<float *>(hist), *f2 = f1 + cap;
+        if (!slot_clear) {
+            __syncthreads();  // the LDS of the selection is reused below
+            for (int i = tid; i < n / 8; i += kWG)
+                reinterpret_cast<uint4 *>(cell16)[i] = make_uint4(0, 0, 0, 0);
+        }
+        if (tid < kFastRows) {
+            sh[kShW1 + tid] = __float_as_uint(P.W.w1[tid]);
+            sh[kShW2 + tid] = __float_as_uint(P.W.w2[tid]);
+        }
+        if (tid == 0) *lcount = 0;
+        __syncthreads();
+        // ---- every entry marks its row in the cell of its coordinate
+        uint32_t tag[kSlots];  // index | value << 16; all ones: no entry
+        int myrow[kSlots];
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            uint32_t idx, vb;
+            bool have;
+            if (j < 4) {
+                idx = (wI[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                vb = (wV[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                have = w_row >= 0 && (unsigned)(w_first + j) < (unsigned)kb;
+                myrow[j] = w_row;
+            } else {
+                have = tid < kb && D.row < P.W.rows;
+                idx = have ? sel_idx[tid] : 0u;
+                vb = have ? sel_val[tid] : 0u;
+                myrow[j] = D.row;
+            }
+            // +-0 values add nothing and are skipped; idx < n keeps a corrupt index inside
+            have = have && idx < (uint32_t)n && (vb & 0x7fffu) != 0;
+            tag[j] = have ? (idx | vb << 16) : 0xffffffffu;
+            if (have) atomicOr(cell32 + (idx >> 1), (1u << myrow[j]) << ((idx & 1u) * 16));
+        }
+        __syncthreads();
+        // ---- a coordinate named by one row has its sums from that entry; the lowest row of
+        //      the others reserves the coordinate's list
+        const float w1_old = w_row >= 0 ? __uint_as_float(sh[kShW1 + w_row]) : 0.0f;
+        const float w2_old = w_row >= 0 ? __uint_as_float(sh[kShW2 + w_row]) : 0.0f;
+        const float w1_cur = __uint_as_float(sh[kShW1 + D.row]);
+        const float w2_cur = __uint_as_float(sh[kShW2 + D.row]);
+        float z1[kSlots], z2[kSlots];  // the entry's terms, then (owners) the coordinate's sums
+        uint32_t aux[kSlots];  // 0: the coordinate is this entry's alone; else its rows (mask)
+                               // and, for the lowest of them, the list's first cell << 16
+        uint32_t owner = 0;    // bit j: slot j computes the update of its coordinate
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            aux[j] = 0;
+            z1[j] = z2[j] = 0.0f;
+            if (tag[j] != 0xffffffffu) {
+                const uint32_t idx = tag[j] & 0xffffu, row = (uint32_t)myrow[j];
+                const uint32_t mask = cell16[idx];
+                const float v = bf2f(tag[j] >> 16);
+                const float vv = v * v;
+                z1[j] = (j < 4 ? w1_old : w1_cur) * v;
+                z2[j] = (j < 4 ? w2_old : w2_cur) * vv;
+                if (mask == 1u << row) {
+                    z1[j] = 0.0f + z1[j];
+                    z2[j] = 0.0f + z2[j];
+                    owner |= 1u << j;
+                } else {
+                    aux[j] = mask;
+                    if ((mask & ((1u << row) - 1u)) == 0) {
+                        aux[j] |= atomicAdd(lcount, (uint32_t)__popc(mask)) << 16;
+                        owner |= 1u << j;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t listed = *lcount;
+        if (listed > (uint32_t)cap) {
+            // more shared coordinates than the lists hold: the general stage, which takes its
+            // entries in its own order and serves shared coordinates row by row
+            slot_clear = false;
+            load_window(G);
+            window_stage(G);
+            param_stage(G);
+            return;
+        }
+        if (listed != 0) {
+#pragma unroll
+            for (int j = 0; j < kSlots; ++j)
+                if (aux[j] != 0 && ((owner >> j) & 1u) != 0)
+                    cell16[tag[j] & 0xffffu] = (uint16_t)(aux[j] >> 16);
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < kSlots; ++j) {
+                if (aux[j] != 0) {
+                    const uint32_t mask = aux[j] & 0xffffu;
+                    const uint32_t at = (uint32_t)cell16[tag[j] & 0xffffu] +
+                                        (uint32_t)__popc(mask & ((1u << myrow[j]) - 1u));
+                    if (at < (uint32_t)cap) {
+                        f1[at] = z1[j];
+                        f2[at] = z2[j];
+                    }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < kSlots; ++j) {
+                if (aux[j] != 0 && ((owner >> j) & 1u) != 0) {
+                    const uint32_t base = aux[j] >> 16;
+                    const int terms = __popc(aux[j] & 0xffffu);
+                    float s1 = 0.0f, s2 = 0.0f;
+                    for (int r = 0; r < terms; ++r) {
+                        uint32_t at = base + (uint32_t)r;
+                        at = at < (uint32_t)cap ? at : (uint32_t)cap - 1u;
+                        s1 = s1 + f1[at];
+                        s2 = s2 + f2[at];
+                    }
+                    z1[j] = s1;
+                    z2[j] = s2;
+                }
+            }
+        }
+        uint32_t upd[kSlots];  // index | update's bf16 bits << 16; all ones: none
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            upd[j] = 0xffffffffu;
+            if (((owner >> j) & 1u) != 0) {
+                const float u = adam_direction(z1[j], z2[j], P.W.s1, P.W.s2, P.W.eps);
+                upd[j] = (tag[j] & 0xffffu) | f2bf(u) << 16;
+            }
+        }
+        // nobody reads the cells' marks any more (the last readers passed a barrier above, or
+        // there were no lists)
+        const float neg_lr = D.neg_lr;
+        if (D.apply_decay != 0) {
+            // every parameter changes: the updates go to the cells, the dense stage does the rest
+#pragma unroll
+            for (int j = 0; j < kSlots; ++j)
+                if (upd[j] != 0xffffffffu) cell16[upd[j] & 0xffffu] = (uint16_t)(upd[j] >> 16);
+            __syncthreads();
+            param_stage(G);
+            return;
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            *reinterpret_cast<uint4 *>(cell16 + chunk_off<C>(wave, c, lane)) = praw[c].q;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            if (upd[j] != 0xffffffffu) {
+                const uint32_t idx = upd[j] & 0xffffu;
+                const float prod = neg_lr * bf2f(upd[j] >> 16);
+                cell16[idx] = (uint16_t)f2bf(bf2f(cell16[idx]) + prod);
+            }
+        }
+        __syncthreads();
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave2, c, lane2);
+            const uint4 q = *reinterpret_cast<const uint4 *>(cell16 + off);
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            const u4 t = {q.x, q.y, q.z, q.w};
+            __builtin_nontemporal_store(t, reinterpret_cast<u4 *>(p + off));
+        }
+    }
+
+    // General window stage without coordinate cells: for each coordinate range (a multiple of
+    // 512, so a chunk lies inside one range) the sums, then the Adam direction in place of
+    // z1, then the parameter update of the chunks in the range.
+    __device__ __forceinline__ void update_by_ranges(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        WindowView wv;
+        wv.I = D.I + G.col0;
+        wv.V = D.V + G.col0;
+        wv.k = D.k;
+        wv.rows = P.W.rows;
+        wv.cur_row = row_in_lds ? D.row : -1;
+        wv.cur_idx = sel_idx;
+        wv.cur_val = sel_val;
+        wv.w1 = P.W.w1;
+        wv.w2 = P.W.w2;
+        __syncthreads();  // the LDS of the selection is reused below
+        for (int lo = 0; lo < n; lo += P.L.sub_len) {
+            const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+            if (HOLD && holding)
+                accumulate_held(G.kb, lo, hi);
+            else
+                window_accumulate(wv, G.kb, lo, hi, z1, z2);
+            for (int c = tid; c < hi - lo; c += kWG) {
+                float u = 0.0f;
+                if (z1[c] != 0.0f || z2[c] != 0.0f)
+                    u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                z1[c] = R::kBF16 ? bf2f(f2bf(u)) : u;
+            }
+            __syncthreads();
+            // store addresses formed afresh, as in param_stage
+            const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const int off = chunk_off<C>(wave2, c, lane2);
+                if (off >= lo && off < hi && (FULL || off < n)) {
+                    float pv[8];
+                    praw[c].to_float(pv);
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        // the range may end inside the chunk only at the end of the block
+                        const float u = (FULL || off + e < n) ? z1[off - lo + e] : 0.0f;
+                        if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                        const float prod = neg_lr * u;
+                        pv[e] = pv[e] + prod;
+                    }
+                    store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    // The slot cells end up holding the update's bits, 0 where no window row names the
+    // coordinate.  Ends with a barrier.
+    __device__ __forceinline__ void window_stage(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const int kb = G.kb;
+        const int rows = P.W.rows;
+        const TensorDesc &D = G.D;
+        if (!slot_clear) {
+            __syncthreads();  // the LDS of the selection is reused below
+            for (int i = tid; i < P.L.slot_cells * P.L.cell_bytes / 16; i += kWG)
+                reinterpret_cast<uint4 *>(cell16)[i] = make_uint4(0, 0, 0, 0);
+        }
+        if (fast_window(G)) {
+            // Every entry of the window is handled once, kEnt per thread.  The rows that name
+            // a coordinate are first gathered as a bit mask in its slot cell.  A coordinate
+            // named by one row gets its update from that entry alone.  The entries of the
+            // others go to a list; the entry of the lowest row owns the coordinate, hands out
+            // one link cell per later row, the later rows file their list position there by
+            // rank, and the owner adds them up in that order, which is the order of the rows.
+            uint32_t *mcount = sh + kShCounter, *lcount = sh + kShLinks, *scount = sh + kShTies;
+            float *f1 = z1, *f2 = z2;
+            const int cap = P.L.z_cap;
+            uint16_t *mI = coord, *mR = mI + cap, *mM = mR + cap, *link = mM + cap;
+            if (tid < kFastRows) {
+                sh[kShW1 + tid] = __float_as_uint(P.W.w1[tid]);
+                sh[kShW2 + tid] = __float_as_uint(P.W.w2[tid]);
+            }
+            if (tid == 0) *mcount = *lcount = *scount = 0;
+            const int wave_first = __builtin_amdgcn_readfirstlane(wave) * kWave;
+            const int entries = rows * kb;
+            const float rkb = __builtin_amdgcn_rcpf((float)kb);
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kEnt; ++i) {
+                uint32_t tag = 0xffffffffu;  // index | row << 16, all ones: nothing to add
+                if (wave_first + i * kWG < entries) {
+                    const int e = tid + i * kWG;
+                    const int row = entry_row(e, rkb);
+                    if (e < entries) {
+                        uint32_t idx = entI[i], vb = entV[i];
+                        if (row == D.row && row_in_lds) {
+                            idx = sel_idx[e - row * kb];
+                            vb = sel_val[e - row * kb];
+                            entV[i] = vb;
+                        }
+                        // +-0 values add nothing and are skipped (the rows of a fresh window
+                        // are all (index 0, value 0)); idx < n keeps a corrupt index inside
+                        if (idx < (uint32_t)n && (vb & 0x7fffu) != 0) {
+                            tag = idx | (uint32_t)row << 16;
+                            atomicOr(cell32 + (idx >> 1), (1u << row) << ((idx & 1u) * 16));
+                        }
+                    }
+                }
+                entI[i] = tag;
+            }
+            __syncthreads();
+            if (R::kBF16 && P.L.compact) {
+                // Slots instead of lists.  A coordinate named by one row gets its update from
+                // that entry.  The others are served row by row, rows separated by barriers:
+                // the first row to come (the lowest) takes a slot for the coordinate and marks
+                // the cell with bit 15 and the slot, later rows add into the slot's sums, so
+                // these are formed in row order.  At most half as many slots as entries.
+                float *s1 = z1, *s2 = z2;
+                uint16_t *scoord = coord;
+                uint32_t multi = 0;  // bit i: entry i shares its coordinate
+#pragma unroll
+                for (int i = 0; i < kEnt; ++i) {
+                    const uint32_t tag = entI[i];
+                    if (tag != 0xffffffffu) {
+                        const uint32_t idx = tag & 0xffffu, row = tag >> 16;
+                        // a cell that a lower row has already marked is not a single either
+                        if (cell16[idx] == 1u << row) {
+                            const float v = bf2f(entV[i]);
+                            const float a1 = __uint_as_float(sh[kShW1 + row]) * v;
+                            const float vv = v * v;
+                            const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
+                            const float u =
+                                adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                            cell16[idx] = (uint16_t)f2bf(u);
+                        } else {
+                            multi |= 1u << i;
+                        }
+                    }
+                }
+                for (int r = 0; r < rows; ++r) {
+#pragma unroll
+                    for (int i = 0; i < kEnt; ++i) {
+                        const uint32_t tag = entI[i];
+                        if (((multi >> i) & 1u) != 0 && (tag >> 16) == (uint32_t)r) {
+                            const uint32_t idx = tag & 0xffffu;
+                            const float v = bf2f(entV[i]);
+                            const float a1 = __uint_as_float(sh[kShW1 + r]) * v;
+                            const float vv = v * v;
+                            const float a2 = __uint_as_float(sh[kShW2 + r]) * vv;
+                            const uint32_t c = cell16[idx];
+                            if ((c & 0x8000u) == 0) {
+                                const uint32_t slot = atomicAdd(mcount, 1u);
+                                if (slot < (uint32_t)cap) {
+                                    cell16[idx] = (uint16_t)(0x8000u | slot);
+                                    s1[slot] = 0.0f + a1;
+                                    s2[slot] = 0.0f + a2;
+                                    scoord[slot] = (uint16_t)idx;
+                                }
+                            } else {
+                                const uint32_t slot = c & 0x7fffu;
+                                s1[slot] = s1[slot] + a1;
+                                s2[slot] = s2[slot] + a2;
+                            }
+                        }
+                    }
+                    __syncthreads();
+                }
+                const int used = (int)(*mcount < (uint32_t)cap ? *mcount : (uint32_t)cap);
+                for (int sl = tid; sl < used; sl += kWG) {
+                    const float u = adam_direction(s1[sl], s2[sl], P.W.s1, P.W.s2, P.W.eps);
+                    cell16[scoord[sl]] = (uint16_t)f2bf(u);
+                }
+                __syncthreads();
+                return;
+            }
+#pragma unroll
+            for (int i = 0; i < kEnt; ++i) {
+                const uint32_t tag = entI[i];
+                if (tag != 0xffffffffu) {
+                    const uint32_t idx = tag & 0xffffu, row = tag >> 16;
+                    const uint32_t mask = cell16[idx];
+                    const float v = bf2f(entV[i]);
+                    const float a1 = __uint_as_float(sh[kShW1 + row]) * v;
+                    const float vv = v * v;
+                    const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
+                    if (mask == 1u << row) {
+                        const float u =
+                            adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                        if (R::kBF16) {
+                            cell16[idx] = (uint16_t)f2bf(u);
+                        } else {  // fp32: the update keeps its bits in a record of its own,
+                                  // handed out from the top of the list arrays
+                            const uint32_t s = (uint32_t)cap - 1u - atomicAdd(scount, 1u);
+                            f1[s] = u;
+                            cell16[idx] = (uint16_t)(s + 1u);
+                        }
+                    } else {
+                        const uint32_t s = atomicAdd(mcount, 1u);
+                        f1[s] = a1;
+                        f2[s] = a2;
+                        mI[s] = (uint16_t)idx;
+                        mR[s] = (uint16_t)row;
+                        mM[s] = (uint16_t)mask;
+                    }
+                }
+            }
+            __syncthreads();
+            const int listed = (int)(*mcount < (uint32_t)cap ? *mcount : (uint32_t)cap);
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below == 0)
+                    cell16[mI[s]] = (uint16_t)atomicAdd(lcount, (uint32_t)__popc(mask) - 1u);
+            }
+            __syncthreads();
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below != 0) {
+                    const uint32_t at = (uint32_t)cell16[mI[s]] + (uint32_t)__popc(below) - 1u;
+                    if (at < (uint32_t)cap) link[at] = (uint16_t)s;
+                }
+            }
+            __syncthreads();
+            for (int s = tid; s < listed; s += kWG) {
+                const uint32_t mask = mM[s], below = mask & ((1u << mR[s]) - 1u);
+                if (below == 0) {
+                    const uint32_t idx = mI[s], base = cell16[idx];
+                    float s1 = 0.0f + f1[s], s2 = 0.0f + f2[s];
+                    const int later = __popc(mask) - 1;
+                    for (int r = 0; r < later; ++r) {
+                        // a valid window keeps base + r and the link inside the list
+                        uint32_t at = base + (uint32_t)r;
+                        at = at < (uint32_t)cap ? at : (uint32_t)cap - 1u;
+                        uint32_t o = link[at];
+                        o = o < (uint32_t)cap ? o : (uint32_t)cap - 1u;
+                        s1 = s1 + f1[o];
+                        s2 = s2 + f2[o];
+                    }
+                    const float u = adam_direction(s1, s2, P.W.s1, P.W.s2, P.W.eps);
+                    if (R::kBF16) {
+                        cell16[idx] = (uint16_t)f2bf(u);
+                    } else {  // the owner's record has given its sums and takes the update
+                        f1[s] = u;
+                        cell16[idx] = (uint16_t)(s + 1);
+                    }
+                }
+            }
+            __syncthreads();
+        } else {
+            WindowView wv;
+            wv.I = D.I + G.col0;
+            wv.V = D.V + G.col0;
+            wv.k = D.k;
+            wv.rows = rows;
+            wv.cur_row = row_in_lds ? D.row : -1;
+            wv.cur_idx = sel_idx;
+            wv.cur_val = sel_val;
+            wv.w1 = P.W.w1;
+            wv.w2 = P.W.w2;
+            for (int lo = 0; lo < n; lo += P.L.sub_len) {
+                const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
+                window_accumulate(wv, kb, lo, hi, z1, z2);
+                for (int c = tid; c < hi - lo; c += kWG) {
+                    if (z1[c] != 0.0f || z2[c] != 0.0f) {
+                        const float u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                        if (R::kBF16) cell16[lo + c] = (uint16_t)f2bf(u);
+                        else cell32[lo + c] = __float_as_uint(u);
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    // the Adam direction of the 8 coordinates at `off`, as the window stage left it in the cells
+    __device__ __forceinline__ void update8(int off, float (&uv)[8]) const {
+        if (R::kBF16 || P.L.cell_bytes == 2) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(cell16 + off);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            if (R::kBF16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uv[2 * i] = __uint_as_float(w[i] << 16);
+                    uv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                }
+            } else {
+                const float *rec = z1;  // record s holds the update of the coordinate with cell s + 1
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t c = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+                    uv[i] = 0.0f;
+                    if (c != 0) uv[i] = rec[c - 1];
+                }
+            }
+        } else {
+            const uint4 a = *reinterpret_cast<const uint4 *>(cell32 + off);
+            const uint4 b2 = *reinterpret_cast<const uint4 *>(cell32 + off + 4);
+            uv[0] = __uint_as_float(a.x); uv[1] = __uint_as_float(a.y);
+            uv[2] = __uint_as_float(a.z); uv[3] = __uint_as_float(a.w);
+            uv[4] = __uint_as_float(b2.x); uv[5] = __uint_as_float(b2.y);
+            uv[6] = __uint_as_float(b2.z); uv[7] = __uint_as_float(b2.w);
+        }
+    }
+
+    __device__ __forceinline__ void param_stage(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        // the store addresses are formed afresh: kept from the loads, they would sit in
+        // registers (or in scratch) through the whole window stage
+        const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave2, c, lane2);
+            if (FULL || off < n) {
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                update8(off, uv);
+                if (apply_decay) {
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        pv[e] = pv[e] * decay;
+                        if (R::kBF16) pv[e] = bf2f(f2bf(pv[e]));
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    const float prod = neg_lr * uv[e];
+                    pv[e] = pv[e] + prod;
+                }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- alpha > 0 with quantisation blocks inside the block (MA:296-298, 311-316) -------------
+    // quantize_dense replaces quantize: e1 = Q(r) is kept as packed codes with its statistics
+    // (for the update, which adds alpha * Qinv(e1)), and the error feedback that is stored is
+    // Q of r2 = (1 - alpha) * Qinv(e1) with statistics of its own.
+    uint32_t dcodes[C], dstat[C];  // e1 of the chunk; its min | max << 16 (bf16 bits)
+
+    __device__ __forceinline__ void quantize_dense(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        uint8_t *err = G.D.err + (G.e0 >> 1);
+        uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
+        uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float x[8];
+            float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                x[e] = r.val(c, e);
+                if (FULL || off + e < n) {
+                    mn = fmin_raw(mn, x[e]);
+                    mx = fmax_raw(mx, x[e]);
+                }
+            }
+            group_minmax<QL>(mn, mx, ql);
+            const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
+            dstat[c] = mnb | mxb << 16;
+            dcodes[c] = 0;
+            float r2[8];
+            float mn2 = INFINITY, mx2 = -INFINITY;
+            if (FULL || off < n) {
+                const float mnf = bf2f(mnb);
+                const float u = div15(bf2f(mxb) - mnf, d15);
+                float cf[8];
+                codes8(x, mnf, u, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                dcodes[c] = pack_codes(cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    float deq = cf[e] * u;
+                    deq = deq + mnf;
+                    const float keep = P.keep * deq;
+                    r2[e] = to_elem(0.0f + keep);
+                    if (FULL || off + e < n) {
+                        mn2 = fmin_raw(mn2, r2[e]);
+                        mx2 = fmax_raw(mx2, r2[e]);
+                    }
+                }
+            }
+            group_minmax<QL>(mn2, mx2, ql);
+            const uint32_t mn2b = f2bf(mn2), mx2b = f2bf(mx2);
+            if (FULL || off < n) {
+                if ((lane & (ql - 1)) == 0) {
+                    const unsigned qb = (unsigned)off >> q_shift;
+                    mnp[qb] = (uint16_t)mn2b;
+                    mxp[qb] = (uint16_t)mx2b;
+                }
+                const float m2f = bf2f(mn2b);
+                const float u2 = div15(bf2f(mx2b) - m2f, d15);
+                float cf[8];
+                codes8(r2, m2f, u2, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // p = p * decay; u = rne(Adam + alpha * Qinv(e1)); p += -lr * u.  After window_stage.
+    __device__ __forceinline__ void param_stage_dense(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        // the store addresses are formed afresh: kept from the loads, they would sit in
+        // registers (or in scratch) through the whole window stage
+        const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave2, c, lane2);
+            if (FULL || off < n) {
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                update8(off, uv);
+                const float mnf = bf2f(dstat[c] & 0xffffu);
+                const float u = div15(bf2f(dstat[c] >> 16) - mnf, d15);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                    const uint32_t code = (dcodes[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                    float deq = (float)code * u;
+                    deq = deq + mnf;
+                    const float add = P.alpha * deq;
+                    const float ud = to_elem(uv[e] + add);
+                    const float prod = neg_lr * ud;
+                    pv[e] = pv[e] + prod;
+                }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // =========================================================================================
+    // Two-pass route: quantisation blocks of q_span >= block length elements (q_span a
+    // multiple of 8), so a top-k block meets at most two of them and their statistics need
+    // every top-k block they cover.  0 <= alpha < 1 (alpha > 0: MA:296-298, 311-316).
+    //   pass 1: a = g + Qinv(e), top-k, window row; the residual r goes to the gradient
+    //           buffer, its exact min / max per (block, segment) to the workspace
+    //   pass 2: statistics of r from the workspace; e1 = Q(r), d1 = Qinv(e1) in registers;
+    //           u = Adam(window) + alpha * d1; p update; r2 = (1 - alpha) * d1; e = Q(r2)
+    //           (alpha == 0: e = e1, u = Adam(window))
+    // r2 is a non-decreasing function of the code, and the code of the element, so the
+    // statistics of r2 over a quantisation block are r2 at the codes of r's extremes: pass 2
+    // needs no second reduction across blocks.
+    // Segment 0 of a block is its part in the quantisation block of its first element,
+    // segment 1 the rest.  Workspace: 4 floats (min0, max0, min1, max1) per block.
+    // =========================================================================================
+    struct Span {
+        int64_t qb0;  // quantisation block of the block's first element
+        int bnd;      // offset inside the block where the next one starts, INT_MAX if it does not
+    };
+
+    __device__ __forceinline__ Span make_span(const BlockGeo &G) const {
+        const int n = FULL ? C * kRound : G.n;
+        Span S;
+        const int64_t q = P.q_span;
+        S.qb0 = G.e0 / q;
+        const int64_t rel = (S.qb0 + 1) * q - G.e0;
+        S.bnd = rel < n ? (int)rel : 0x7fffffff;
+        return S;
+    }
+
+    __device__ __forceinline__ int64_t block_id(const BlockGeo &G) const {
+        const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
+        return G.e0 / dbs;
+    }
+
+    // min / max over the workgroup of two pairs; every thread gets the result.  Uses the 32
+    // words at kShW1 and three barriers.
+    __device__ __forceinline__ void wg_minmax2(float (&mn)[2], float (&mx)[2]) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) group_minmax<0>(mn[s2], mx[s2], kWave);
+        __syncthreads();
+        if (lane == 0) {
+            sh[kShW1 + wave * 4 + 0] = __float_as_uint(mn[0]);
+            sh[kShW1 + wave * 4 + 1] = __float_as_uint(mx[0]);
+            sh[kShW1 + wave * 4 + 2] = __float_as_uint(mn[1]);
+            sh[kShW1 + wave * 4 + 3] = __float_as_uint(mx[1]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mn[0] = fmin_raw(mn[0], __uint_as_float(sh[kShW1 + w * 4 + 0]));
+            mx[0] = fmax_raw(mx[0], __uint_as_float(sh[kShW1 + w * 4 + 1]));
+            mn[1] = fmin_raw(mn[1], __uint_as_float(sh[kShW1 + w * 4 + 2]));
+            mx[1] = fmax_raw(mx[1], __uint_as_float(sh[kShW1 + w * 4 + 3]));
+        }
+        __syncthreads();  // the words are free again
+    }
+
+    __device__ __forceinline__ void store_partials(const BlockGeo &G, float (&mn)[2],
+                                                   float (&mx)[2]) {
+        wg_minmax2(mn, mx);
+        if (tid == 0)
+            *reinterpret_cast<float4 *>(G.D.ws + block_id(G) * 4) =
+                make_float4(mn[0], mx[0], mn[1], mx[1]);
+    }
+
+    // exact min / max of r over the two quantisation blocks this top-k block meets, from the
+    // partials of all top-k blocks that cover them (at most 64 each: lane i takes one)
+    __device__ __forceinline__ void gather_extremes(const BlockGeo &G, const Span &S,
+                                                    float (&mnx)[2], float (&mxx)[2]) const {
+        const int64_t q = P.q_span;
+        const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
+        const int64_t nblk = (G.D.d + dbs - 1) / dbs;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            float mn = INFINITY, mx = -INFINITY;
+            if (s2 == 0 || S.bnd != 0x7fffffff) {
+                const int64_t Q = S.qb0 + s2;
+                const int64_t first = Q * q;
+                const int64_t b_lo = first / dbs;
+                int64_t b_hi = (first + q - 1) / dbs;
+                b_hi = b_hi < nblk - 1 ? b_hi : nblk - 1;
+                const int64_t b = b_lo + lane;
+                if (b <= b_hi) {
+                    const int seg = b * dbs >= first ? 0 : 1;
+                    const float *w = G.D.ws + b * 4 + seg * 2;
+                    mn = w[0];
+                    mx = w[1];
+                }
+                group_minmax<0>(mn, mx, kWave);
+            }
+            mnx[s2] = mn;
+            mxx[s2] = mx;
+        }
+    }
+
+    // Statistics of r (sp_mn / sp_mx) and of r2 (sp2_mn / sp2_mx) for both segments, from the
+    // exact extremes of r.
+    template <bool DENSE>
+    __device__ __forceinline__ void span_statistics(const BlockGeo &G, const Span &S) {
+        float mnx[2], mxx[2];
+        gather_extremes(G, S, mnx, mxx);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            sp_mn[s2] = f2bf(mnx[s2]);
+            sp_mx[s2] = f2bf(mxx[s2]);
+            if (!DENSE) {  // alpha == 0: e = Q(r), the statistics kept are r's
+                sp2_mn[s2] = sp_mn[s2];
+                sp2_mx[s2] = sp_mx[s2];
+                continue;
+            }
+            const float mnf = bf2f(sp_mn[s2]);
+            const float u = div15(bf2f(sp_mx[s2]) - mnf, d15);
+            float x[8], cf[8];
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) x[e] = (e & 1) ? mxx[s2] : mnx[s2];
+            codes8(x, mnf, u, cf);
+            float lo = cf[0] * u, hi = cf[1] * u;
+            lo = lo + mnf;
+            hi = hi + mnf;
+            lo = P.keep * lo;
+            hi = P.keep * hi;
+            sp2_mn[s2] = f2bf(to_elem(0.0f + lo));
+            sp2_mx[s2] = f2bf(to_elem(0.0f + hi));
+        }
+    }
+
+    // 4-bit codes of 8 values against (mn, u) as small exact floats: floor((x - mn)/u + 0.5)
+    // clamped to [0, 15]; all zero when the range is zero or not finite.  Same arithmetic as
+    // the quantize stage.
+    __device__ __forceinline__ void codes8(const float (&x)[8], float mnf, float u,
+                                           float (&cf)[8]) const {
+        const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
+        const float lim = 32.0f * u;
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            y[e] = x[e] - mnf;
+            if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
+        }
+        if constexpr (R::kBF16) {
+            // Short way.  With q the exact quotient y / u, both the correctly rounded quotient
+            // and y * rcp(u) (rcp is within one ulp) lie within 2^-19 of q for q < 16.5, and the
+            // sum with 0.5 rounds by at most 2^-20 more: wherever y * rcp(u) stays 2^-16 away
+            // from every k + 0.5, rounding it to the nearest integer gives floor(y / u + 0.5) as
+            // the long way computes it.  bf16 data lies inside its exact statistics, so the
+            // result is in [0, 15].  A wave with an element too close to call, or with a step
+            // outside the comfortable exponent range, goes the long way (one element in 2^15).
+            const float r0 = __builtin_amdgcn_rcpf(u);
+            float far = 0.0f;
+#pragma unroll
+            for (int e = 0; e < kChunk; e += 2) {
+                const float q0 = y[e] * r0, q1 = y[e + 1] * r0;
+                cf[e] = __builtin_rintf(q0);
+                cf[e + 1] = __builtin_rintf(q1);
+                const float d0 = q0 - cf[e], d1 = q1 - cf[e + 1];
+                asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(far) : "v"(far), "v"(d0), "v"(d1));
+            }
+            const bool fine = ex - 32u <= 190u && far <= 0.5f - 0x1p-16f;
+            if (__builtin_amdgcn_ballot_w64(!fine) == 0) return;
+        }
+        bool ok = true;
+        float us = u;
+        if (ex - 32u > 190u) {
+            ok = u != 0.0f && isfinite(u);
+            const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
+            us = ok ? u * sc : 1.0f;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
+        }
+        const Divisor dv = make_divisor(us);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            float v = div_shared(y[e], dv);
+            v = floorf(v + 0.5f);
+            cf[e] = v;
+        }
+        // bf16 data lies inside its exact statistics, so its codes need no clamp unless the
+        // step itself is so small that it was rounded coarsely
+        if (!R::kBF16 || ex - 32u > 190u) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const float v = __builtin_amdgcn_fmed3f(cf[e], 0.0f, 15.0f);
+                cf[e] = ok ? v : 0.0f;
+            }
+        }
+    }
+
+    // two 16-bit halves, nibble order (e0 e1)(e2 e3) | (e4 e5)(e6 e7), even element high
+    static __device__ __forceinline__ uint32_t pack_codes(const float (&cf)[8]) {
+        float lo = cf[2];
+        lo = __builtin_fmaf(lo, 16.0f, cf[3]);
+        lo = __builtin_fmaf(lo, 16.0f, cf[0]);
+        lo = __builtin_fmaf(lo, 16.0f, cf[1]);
+        float hi = cf[6];
+        hi = __builtin_fmaf(hi, 16.0f, cf[7]);
+        hi = __builtin_fmaf(hi, 16.0f, cf[4]);
+        hi = __builtin_fmaf(hi, 16.0f, cf[5]);
+        return (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+
+    static __device__ __forceinline__ float to_elem(float v) {
+        return R::kBF16 ? bf2f(f2bf(v)) : v;
+    }
+
+    // ---- pass 1 ------------------------------------------------------------------------------
+    uint32_t sp_mn[2], sp_mx[2];    // statistics of r in the two segments (bf16 bits)
+    uint32_t sp2_mn[2], sp2_mx[2];  // statistics of r2
+
+    __device__ __forceinline__ void span_load_grad_inputs(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+        const uint8_t *err = G.D.err + (G.e0 >> 1);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            graw[c].load(g, off, n, FULL);
+            cw[c] = 0;
+            if (FULL || off < n) {
+                if (FULL || off + kChunk <= n) {
+                    cw[c] = *reinterpret_cast<const uint32_t *>(err + ((unsigned)off >> 1));
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        cw[c] |= (uint32_t)err[(off >> 1) + j] << (8 * j);
+                }
+            }
+        }
+        sp_mn[0] = G.D.mn[S.qb0];
+        sp_mx[0] = G.D.mx[S.qb0];
+        sp_mn[1] = sp_mx[1] = 0;
+        if (S.bnd != 0x7fffffff) {
+            sp_mn[1] = G.D.mn[S.qb0 + 1];
+            sp_mx[1] = G.D.mx[S.qb0 + 1];
+        }
+    }
+
+    __device__ __forceinline__ void span_dequant(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            float v[8];
+            graw[c].to_float(v);
+            const bool second = off >= S.bnd;
+            const float mn = second ? mn1 : mn0, u = second ? u1 : u0;
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                float deq = (float)code * u;
+                deq = deq + mn;
+                v[e] = v[e] + deq;
+            }
+            if (!FULL && off + kChunk > n) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (off + e >= n) v[e] = 0.0f;
+            }
+            r.set_chunk(c, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        launder(r);
+    }
+
+    // the residual goes to the gradient buffer (which the step may destroy, MA:190-214 does)
+    __device__ __forceinline__ void span_store_residual(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        elem_t *out = reinterpret_cast<elem_t *>(const_cast<void *>(G.D.g)) + G.e0;
+        float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float x[8];
+                float lmn = INFINITY, lmx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    x[e] = r.val(c, e);
+                    if (FULL || off + e < n) {
+                        lmn = fmin_raw(lmn, x[e]);
+                        lmx = fmax_raw(lmx, x[e]);
+                    }
+                }
+                const bool second = off >= S.bnd;
+                mn[0] = fmin_raw(mn[0], second ? INFINITY : lmn);
+                mx[0] = fmax_raw(mx[0], second ? -INFINITY : lmx);
+                mn[1] = fmin_raw(mn[1], second ? lmn : INFINITY);
+                mx[1] = fmax_raw(mx[1], second ? lmx : -INFINITY);
+                store8(out, off, FULL ? 0x7fffffff : n, true, x);
+            }
+        }
+        store_partials(G, mn, mx);
+    }
+
+    // ---- pass 2 -----------------------------------------------------------------------
+    __device__ __forceinline__ void span_load_residual(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) graw[c].load(g, chunk_off<C>(wave, c, lane), n, FULL);
+    }
+
+    // alpha == 0, second pass: e = Q(r) against the statistics of r, and the statistics arrays
+    __device__ __forceinline__ void span_codes_stage(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        uint8_t *err = D.err + (G.e0 >> 1);
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                const bool second = off >= S.bnd;
+                float x[8], cf[8];
+                graw[c].to_float(x);
+                codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+        }
+        span_store_statistics(G, S);
+    }
+
+    // the block that holds the first element of a quantisation block writes its statistics
+    __device__ __forceinline__ void span_store_statistics(const BlockGeo &G, const Span &S) {
+        if (tid == 0) {
+            if (G.e0 == S.qb0 * (int64_t)P.q_span) {
+                G.D.mn[S.qb0] = (uint16_t)sp2_mn[0];
+                G.D.mx[S.qb0] = (uint16_t)sp2_mx[0];
+            }
+            if (S.bnd != 0x7fffffff) {
+                G.D.mn[S.qb0 + 1] = (uint16_t)sp2_mn[1];
+                G.D.mx[S.qb0 + 1] = (uint16_t)sp2_mx[1];
+            }
+        }
+    }
+
+    // alpha > 0, second pass: p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
+    // r2 = rne(0 + keep * d1); e = Q(r2); the statistics arrays.  After window_stage.
+    __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        const TensorDesc &D = G.D;
+        elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
+        uint8_t *err = D.err + (G.e0 >> 1);
+        const float neg_lr = D.neg_lr, decay = D.decay;
+        const bool apply_decay = D.apply_decay != 0;
+        const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
+        const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
+        const float m20 = bf2f(sp2_mn[0]), m21 = bf2f(sp2_mn[1]);
+        const float v0 = div15(bf2f(sp2_mx[0]) - m20, d15), v1 = div15(bf2f(sp2_mx[1]) - m21, d15);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                const bool second = off >= S.bnd;
+                float x[8], cf[8], d1[8];
+                graw[c].to_float(x);
+                codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
+                const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    float deq = cf[e] * u;
+                    d1[e] = deq + mnf;
+                }
+                float pv[8], uv[8];
+                praw[c].to_float(pv);
+                update8(off, uv);
+                float r2[8];
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (apply_decay) pv[e] = to_elem(pv[e] * decay);
+                    const float add = P.alpha * d1[e];
+                    const float ud = to_elem(uv[e] + add);
+                    const float prod = neg_lr * ud;
+                    pv[e] = pv[e] + prod;
+                    const float keep = P.keep * d1[e];
+                    r2[e] = to_elem(0.0f + keep);
+                }
+                store8(p, off, FULL ? 0x7fffffff : n, true, pv);
+                codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e)
+                    if (!FULL && off + e >= n) cf[e] = 0.0f;
+                const uint32_t codes = pack_codes(cf);
+                if (FULL || off + kChunk <= n) {
+                    *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
+                } else {
+                    const int nbytes = (n - off + 1) >> 1;
+                    for (int j = 0; j < nbytes; ++j)
+                        err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        span_store_statistics(G, S);
+    }
+};
+
+// Work item of this workgroup.  The hardware hands consecutive workgroups of a launch to the
+// chip's 8 XCDs in turn (workgroup i runs on XCD i % 8, each with its own L2); the items are
+// dealt out so that every XCD walks one contiguous eighth of the launch's blocks, which the
+// memory system serves measurably faster than eight interleaved walks (stores most of all).
+__device__ __forceinline__ int xcd_contiguous_item(int total_items) {
+    constexpr int kXcds = 8;
+    const int bid = (int)blockIdx.x;
+    const int x = bid % kXcds, j = bid / kXcds;
+    const int q = total_items / kXcds, r = total_items % kXcds;
+    return x * q + (x < r ? x : r) + j;
+}
+
+// which tensor owns workgroup / work item `w` of the launch (first_block is ascending)
+__device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
+    // the last tensor whose first work item is not beyond w
+    int lo = 0, hi = P.n_tensors - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (w >= P.t[mid].first_block) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+// One workgroup per block: any block shape.  Tensor i contributes its blocks
+// blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
+template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+#ifdef MA_EXP_NOREMAP
+    const int item = (int)blockIdx.x;
+#else
+    const int item = xcd_contiguous_item(P.total_items);
+#endif
+    const int ti = find_tensor(P, item);
+    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
+    auto run = [&](auto &fb) {
+        fb.load_grad_inputs(G);
+        fb.dequant(G);
+        // the older window rows are most of this path's traffic: asked for before the selection
+        if constexpr (HOLD) fb.load_held(G, false);
+#ifdef MA_EXP_SKIP_TOPK
+        if (threadIdx.x < G.kb) { fb.sel_idx[threadIdx.x] = threadIdx.x; fb.sel_val[threadIdx.x] = 0; }
+        __syncthreads();
+#else
+        fb.topk_and_row(G);
+#endif
+#ifdef MA_EXP_SKIP_QUANT
+        launder(fb.r);
+        fb.load_params_window(G);
+        fb.update(G);
+        return;
+#endif
+#ifdef MA_EXP_SKIP_UPDATE
+        fb.quantize(G);
+        return;
+#endif
+#ifdef MA_EXP_SKIP_WINDOW
+        fb.quantize(G);
+        fb.load_params_window(G);
+        fb.param_stage(G);
+        return;
+#endif
+        if constexpr (DENSE) {
+            fb.quantize_dense(G);
+            fb.load_params(G);
+            fb.load_window(G);
+            fb.window_stage(G);
+            fb.param_stage_dense(G);
+        } else {
+            fb.quantize(G);
+            // asked for only now: measured faster than at the start of the block, where they
+            // keep 30 more registers live through the selection and the quantisation
+            fb.load_params_window(G);
+            if constexpr (HOLD) fb.load_held(G, true);
+            fb.update(G);
+        }
+    };
+    if (G.n == R::kC * kRound) {
+        FusedBlock<R, true, QL, HOLD> fb(P, lds);
+        run(fb);
+    } else {
+        FusedBlock<R, false, QL, HOLD> fb(P, lds);
+        run(fb);
+    }
+}
+
+// Two-pass route, see FusedBlock; one workgroup per block.
+//   alpha > 0:  PASS 1 (residual and its extremes), PASS 2 (everything else)
+//   alpha == 0: PASS 4 (PASS 1 and the parameter update, which does not wait for the
+//               statistics), PASS 3 (codes of the residual)
+template <class R, int MIN_WAVES, int PASS>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+#ifdef MA_EXP_NOREMAP
+    const int item = (int)blockIdx.x;
+#else
+    const int item = xcd_contiguous_item(P.total_items);
+#endif
+    const int ti = find_tensor(P, item);
+    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
+    auto run = [&](auto &fb) {
+        const auto S = fb.make_span(G);
+        if constexpr (PASS == 1 || PASS == 4) {
+            fb.span_load_grad_inputs(G, S);
+            fb.span_dequant(G, S);
+            fb.topk_and_row(G);
+            fb.span_store_residual(G, S);
+            if constexpr (PASS == 4) {
+                fb.load_params_window(G);
+                fb.update(G);
+            }
+        } else if constexpr (PASS == 2) {
+            fb.row_in_lds = false;
+            fb.load_window(G);
+            fb.span_load_residual(G);
+            fb.template span_statistics<true>(G, S);
+            fb.load_params(G);
+            fb.window_stage(G);
+            fb.span_param_stage(G, S);
+        } else {
+            fb.span_load_residual(G);
+            fb.template span_statistics<false>(G, S);
+            fb.span_codes_stage(G, S);
+        }
+    };
+    if (G.n == R::kC * kRound) {
+        FusedBlock<R, true, 0> fb(P, lds);
+        run(fb);
+    } else {
+        FusedBlock<R, false, 0> fb(P, lds);
+        run(fb);
+    }
+}
+
+// =============================================================================================
+// Launchers
+// =============================================================================================
+
+constexpr int kLdsLimit = 160 * 1024;
+
+static inline int launch_status() { return (int)hipGetLastError(); }
+
+
+template <class K>
+static int allow_big_lds(K kernel, int bytes) {
+    if (bytes <= 64 * 1024) return 0;
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+constexpr int kWavesThreeWG = 3 * kWG / 256;  // three workgroups per CU
+constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
+
+template <class R, int QL, bool DENSE = false, bool HOLD = false>
+static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    // bf16 blocks of up to 20480 elements fit 80 registers and a third of the LDS: three
+    // workgroups per CU; the general window stage with the window held in registers takes the
+    // budget of two
+    constexpr int kWaves_ =
+        (R::kBF16 && R::kC <= kClass2 && !HOLD) ? kWavesThreeWG : kMinWaves;
+    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD>, lds_bytes);
+    if (rc) return rc;
+    fused_step_kernel<R, kWaves_, QL, DENSE, HOLD><<<grid, kWG, lds_bytes, s>>>(P);
+    return launch_status();
+}
+
+// alpha > 0
+template <template <int> class RT>
+static int launch_fused_dense(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                              const FusedParams &P) {
+    if (C == kClass2 && P.q_shift == 6)
+        return launch_fused_one<RT<kClass2>, 8, true>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 5)
+        return launch_fused_one<RT<kClass2>, 4, true>(grid, lds_bytes, s, P);
+    switch (C) {
+        case kClass0: return launch_fused_one<RT<kClass0>, 0, true>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0, true>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0, true>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0, true>(grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
+}
+
+template <template <int> class RT>
+static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    // the hardware-sized block gets kernels with the quantisation group size compiled in
+    if constexpr (RT<kClass2>::kBF16) {
+        // windows too large for the one-pass stage: the general stage, window in registers
+        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 6)
+            return launch_fused_one<RT<kClass2>, 8, false, true>(grid, lds_bytes, s, P);
+        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 5)
+            return launch_fused_one<RT<kClass2>, 4, false, true>(grid, lds_bytes, s, P);
+    }
+    if (C == kClass2 && P.q_shift == 6) return launch_fused_one<RT<kClass2>, 8>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 5) return launch_fused_one<RT<kClass2>, 4>(grid, lds_bytes, s, P);
+    switch (C) {
+        case kClass0: return launch_fused_one<RT<kClass0>, 0>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0>(grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
+}
+
+template <class R>
+static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                           const FusedParams &P) {
+    // the first pass has the register needs of the fused kernel
+    constexpr int kFirst = (R::kBF16 && R::kC <= kClass2) ? kWavesThreeWG : kMinWaves;
+    int rc;
+    switch (pass) {
+        case 1:
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 1>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kFirst, 1><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        case 2:
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 2>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kFirst, 2><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        case 4:
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 4>, lds_bytes);
+            if (rc) return rc;
+            span_step_kernel<R, kFirst, 4><<<grid, kWG, lds_bytes, s>>>(P);
+            break;
+        default:  // needs the kSh* words only
+            span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
+            break;
+    }
+    return launch_status();
+}
+
+template <template <int> class RT>
+static int launch_span(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                       const FusedParams &P) {
+    switch (C) {
+        case kClass0: return launch_span_one<RT<kClass0>>(pass, grid, lds_bytes, s, P);
+        case kClass1: return launch_span_one<RT<kClass1>>(pass, grid, lds_bytes, s, P);
+        case kClass2: return launch_span_one<RT<kClass2>>(pass, grid, lds_bytes, s, P);
+        case kClass3: return launch_span_one<RT<kClass3>>(pass, grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
+}
+
+// The instantiations, one translation unit each.
+int launch_fused_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
+int launch_fused_f32(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
+int launch_fused_dense_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                            const FusedParams &P);
+int launch_fused_dense_f32(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                           const FusedParams &P);
+int launch_span_bf16(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                     const FusedParams &P);
+int launch_span_f32(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                    const FusedParams &P);
+
+}  // namespace ma

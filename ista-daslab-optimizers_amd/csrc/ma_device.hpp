@@ -12,19 +12,16 @@
 
 namespace ma {
 
-#ifndef MA_WG
-#define MA_WG 512  // threads per workgroup of the block kernels: 256 or 512
-#endif
-constexpr int kWG = MA_WG;
+constexpr int kWG = 512;  // threads per workgroup of the block kernels
 constexpr int kWave = 64;
 constexpr int kWaves = kWG / kWave;
 constexpr int kChunk = 8;        // elements per lane per chunk
 constexpr int kRound = kWG * kChunk;  // elements one chunk of every thread covers together
 // register-tile classes: chunks per thread for blocks up to 4096 / ~10-12 K / 20480 / 32768
-constexpr int kClass0 = kWG == 256 ? 2 : 1;
-constexpr int kClass1 = kWG == 256 ? 5 : 3;
-constexpr int kClass2 = kWG == 256 ? 10 : 5;
-constexpr int kClass3 = kWG == 256 ? 16 : 8;
+constexpr int kClass0 = 1;
+constexpr int kClass1 = 3;
+constexpr int kClass2 = 5;
+constexpr int kClass3 = 8;
 // words of the small LDS scratch every block kernel has at offset 0
 constexpr int kShScan = 0;      // 8 words: per-wave partial sums
 constexpr int kShCounter = 8;   // slot allocation counter of the window pass
@@ -40,30 +37,6 @@ constexpr int kShW1 = 32;       // 16 words: beta1^age of the window rows
 constexpr int kShW2 = 48;       // 16 words: beta2^age of the window rows
 constexpr int kHistCopies = 32;  // LDS histogram replicas, one per bank
 constexpr int kMaxWindow = 64;
-
-// ---- development aid ---------------------------------------------------------------------------
-// With MA_PHASE_TIMING (never defined in the shipped build) thread 0 of every workgroup adds
-// the cycles between marks into a caller-provided buffer; otherwise the timer is empty.
-#ifdef MA_PHASE_TIMING
-__device__ unsigned long long *g_phase_buf = nullptr;
-struct PhaseTimer {
-    unsigned long long t;
-    __device__ __forceinline__ void begin() { t = __builtin_readcyclecounter(); }
-    __device__ __forceinline__ void mark(int i) {
-        if (threadIdx.x == 0 && g_phase_buf) {
-            const unsigned long long now = __builtin_readcyclecounter();
-            atomicAdd(&g_phase_buf[i], now - t);
-            t = now;
-        }
-    }
-};
-#else
-struct PhaseTimer {
-    __device__ __forceinline__ void begin() {}
-    // leaves a comment in the assembly listing so that instruction counts can be read per phase
-    __device__ __forceinline__ void mark(int i) { asm volatile("; phase mark %0" ::"n"(i)); }
-};
-#endif
 
 // The thread id as a value the optimiser cannot see through.  The selection helpers derive
 // their lane offsets from this, so that the offsets are rebuilt where they are used instead
@@ -327,8 +300,7 @@ __device__ __forceinline__ void launder(R &r) {
 //   hist: 257 << copies_log2 words (bin 256 is a discard bin), sh: 8 words.  Ends with a barrier.
 template <class R>
 __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, uint32_t *sh,
-                                                 uint32_t &T, int &take_eq, PhaseTimer &pt,
-                                                 int pt0, int copies_log2) {
+                                                 uint32_t &T, int &take_eq, int copies_log2) {
     const int copies = 1 << copies_log2;
     constexpr int kPasses = R::kBF16 ? 2 : 4;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
@@ -343,7 +315,6 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
         for (int i = tid; i < (nb + 1) * copies; i += kWG) hist[i] = 0;
         launder(r);
         __syncthreads();
-        if (pass < 2) pt.mark(pt0 + 3 * pass);
 #pragma unroll
         for (int c = 0; c < R::kC; ++c) {
 #pragma unroll
@@ -356,7 +327,6 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
             __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
-        if (pass < 2) pt.mark(pt0 + 3 * pass + 1);
         // thread tid owns bin nb-1-tid so that a forward scan walks the bins from the top
         const int bin = nb - 1 - tid;
         uint32_t cnt = 0;
@@ -374,7 +344,6 @@ __device__ __forceinline__ void select_threshold(R &r, int kb, uint32_t *hist, u
         prefix |= sh[kShPivot] << shift;
         pmask |= dm << shift;
         need = (int)sh[kShNeed];
-        if (pass < 2) pt.mark(pt0 + 3 * pass + 2);
     }
     __syncthreads();
     T = prefix;
@@ -485,7 +454,7 @@ constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multi
 template <class R>
 __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uint32_t *hist,
                                                uint32_t *sh, uint16_t *sel_idx,
-                                               uint16_t *sel_val, PhaseTimer &pt) {
+                                               uint16_t *sel_val) {
     constexpr int C = R::kC;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t *cand = hist + 2 * kSmallHistWords;
@@ -501,7 +470,6 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         cmax[c] = chunk_max_key(r.w[c]);
     }
     __syncthreads();
-    pt.mark(1);
     int unused_take, unused_eq;
     // one key per thread: the largest of its chunk maxima
     uint32_t tmax[1] = {cmax[0]};
@@ -509,7 +477,6 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     for (int c = 1; c < C; ++c) tmax[0] = cmax[c] > tmax[0] ? cmax[c] : tmax[0];
     const uint32_t L = select_kth_key15<1>(tmax, 1u, kb, hist, sh + kShSel, sh + kShNEq,
                                            unused_take, unused_eq);
-    pt.mark(2);
 
     // candidates: every element with key >= L, wave by wave into the wave's own list
     uint32_t todo = 0;
@@ -548,7 +515,6 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     if (lane < 16 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
     if (lane == 0) sh[kShCnts + wave] = filled;
     __syncthreads();
-    pt.mark(3);
     uint32_t cnts[kWaves];
     bool ok = true;
 #pragma unroll
@@ -620,7 +586,6 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         }
         __syncthreads();
     }
-    pt.mark(4);
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         const int off = chunk_off<C>(wave, c, lane);
@@ -642,7 +607,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
 template <class R>
 __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, int kb,
                                                  uint16_t *sel_idx, uint16_t *sel_val,
-                                                 uint32_t *sh, PhaseTimer &pt, int pt0) {
+                                                 uint32_t *sh) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     uint32_t pre[R::kC];  // low 16: entries >= T before this lane's chunk; high 16: == T
     uint32_t run = 0;
@@ -666,7 +631,6 @@ __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, 
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
         if (w < wave) base += sh[w];
-    pt.mark(pt0);
 #pragma unroll
     for (int c = 0; c < R::kC; ++c) {
         uint32_t p = pre[c] + base;
@@ -691,7 +655,6 @@ __device__ __forceinline__ void compact_selected(R &r, uint32_t T, int take_eq, 
         __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
-    pt.mark(pt0 + 1);
 }
 
 // ---- Adam statistics of one block from its window rows ---------------------------------------------
