@@ -378,8 +378,23 @@ struct FusedBlock {
         return (int)(((float)e + 0.5f) * rkb);
     }
 
+    // ---- a lower bound for this step's selection threshold: the magnitudes of the entries the
+    //      previous step took from this block (hint_topk_bf16 tries the smallest, lowered a little)
+    uint32_t hint;
+
+    __device__ __forceinline__ void load_hint(const BlockGeo &G) {
+        hint = 0x7fffu;
+        if constexpr (FULL && R::kBF16) {
+            if (tid < G.kb && G.kb <= kWG) {
+                const int prev = (G.D.row == 0 ? P.W.rows_total : G.D.row) - 1;
+                hint = G.D.V[(int64_t)prev * G.D.k + G.col0 + tid] & 0x7fffu;
+            }
+        }
+    }
+
     // ---- gradient, 4-bit error feedback and its statistics
     __device__ __forceinline__ void load_grad_inputs(const BlockGeo &G) {
+        load_hint(G);
         const int n = FULL ? C * kRound : G.n;
         const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
         const uint8_t *err = G.D.err + (G.e0 >> 1);
@@ -443,9 +458,11 @@ struct FusedBlock {
             }
             const float mn = bf2f(mnb), mx = bf2f(mxb);
             const float u = div15(mx - mn, d15);
+            // the nibbles as bytes of two words (even elements high), one conversion each
+            const uint32_t odd = cw[c] & 0x0f0f0f0fu, even = (cw[c] >> 4) & 0x0f0f0f0fu;
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                const uint32_t code = (((e & 1) ? odd : even) >> (8 * (e >> 1))) & 0xffu;
                 float deq = (float)code * u;
                 deq = deq + mn;
                 v[e] = v[e] + deq;
@@ -467,7 +484,11 @@ struct FusedBlock {
         bool topk_done = false;
         if constexpr (FULL && R::kBF16) {
             if (kb <= kWG) {
-                topk_done = fast_topk_bf16(r, kb, cell16, hist, sh, sel_idx, sel_val);
+                topk_done = hint_topk_bf16(r, kb, hint, cell16, hist, sh, sel_idx, sel_val);
+#ifndef MA_EXP_NOFALLBACK
+                if (!topk_done)
+                    topk_done = fast_topk_bf16(r, kb, cell16, hist, sh, sel_idx, sel_val);
+#endif
                 launder(r);
                 // the block was parked in the slot cells and every thread cleared its own
                 slot_clear = topk_done && P.L.slot_cells == C * kRound;
@@ -1383,58 +1404,31 @@ struct FusedBlock {
     // the quantize stage.
     __device__ __forceinline__ void codes8(const float (&x)[8], float mnf, float u,
                                            float (&cf)[8]) const {
-        const uint32_t ex = (__float_as_uint(u) >> 23) & 0xffu;
         const float lim = 32.0f * u;
         float y[8];
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
             y[e] = x[e] - mnf;
+            // fp32 data may leave the bf16-rounded range; anything beyond +-32 u clamps to an
+            // end code either way
             if (!R::kBF16) y[e] = __builtin_amdgcn_fmed3f(y[e], -lim, lim);
         }
-        if constexpr (R::kBF16) {
-            // Short way.  With q the exact quotient y / u, both the correctly rounded quotient
-            // and y * rcp(u) (rcp is within one ulp) lie within 2^-19 of q for q < 16.5, and the
-            // sum with 0.5 rounds by at most 2^-20 more: wherever y * rcp(u) stays 2^-16 away
-            // from every k + 0.5, rounding it to the nearest integer gives floor(y / u + 0.5) as
-            // the long way computes it.  bf16 data lies inside its exact statistics, so the
-            // result is in [0, 15].  A wave with an element too close to call, or with a step
-            // outside the comfortable exponent range, goes the long way (one element in 2^15).
-            const float r0 = __builtin_amdgcn_rcpf(u);
-            float far = 0.0f;
-#pragma unroll
-            for (int e = 0; e < kChunk; e += 2) {
-                const float q0 = y[e] * r0, q1 = y[e + 1] * r0;
-                cf[e] = __builtin_rintf(q0);
-                cf[e + 1] = __builtin_rintf(q1);
-                const float d0 = q0 - cf[e], d1 = q1 - cf[e + 1];
-                asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(far) : "v"(far), "v"(d0), "v"(d1));
-            }
-            const bool fine = ex - 32u <= 190u && far <= 0.5f - 0x1p-16f;
-            if (__builtin_amdgcn_ballot_w64(!fine) == 0) return;
-        }
-        bool ok = true;
-        float us = u;
-        if (ex - 32u > 190u) {
-            ok = u != 0.0f && isfinite(u);
-            const float sc = ex < 32u ? 0x1p64f : 0x1p-64f;
-            us = ok ? u * sc : 1.0f;
-#pragma unroll
-            for (int e = 0; e < kChunk; ++e) y[e] = y[e] * sc;
-        }
-        const Divisor dv = make_divisor(us);
-#pragma unroll
-        for (int e = 0; e < kChunk; ++e) {
-            float v = div_shared(y[e], dv);
-            v = floorf(v + 0.5f);
-            cf[e] = v;
-        }
-        // bf16 data lies inside its exact statistics, so its codes need no clamp unless the
-        // step itself is so small that it was rounded coarsely
-        if (!R::kBF16 || ex - 32u > 190u) {
+        if (divisor_is_plain(u)) {
+            const Divisor dv = make_divisor(u);
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                const float v = __builtin_amdgcn_fmed3f(cf[e], 0.0f, 15.0f);
-                cf[e] = ok ? v : 0.0f;
+                const float v = floorf(div_shared(y[e], dv) + 0.5f);
+                // bf16 data lies inside its exact statistics: no clamp needed
+                cf[e] = R::kBF16 ? v : __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+            }
+        } else {
+            // a step that is zero, not finite, tiny, huge or has an all-ones significand: the
+            // compiler's division; with so coarse a step even bf16 data can leave [0, 15]
+            const bool ok = u != 0.0f && isfinite(u);
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                const float v = floorf(y[e] / u + 0.5f);
+                cf[e] = ok ? __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f) : 0.0f;
             }
         }
     }
@@ -1461,6 +1455,7 @@ struct FusedBlock {
     uint32_t sp2_mn[2], sp2_mx[2];  // statistics of r2
 
     __device__ __forceinline__ void span_load_grad_inputs(const BlockGeo &G, const Span &S) {
+        load_hint(G);
         const int n = FULL ? C * kRound : G.n;
         const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
         const uint8_t *err = G.D.err + (G.e0 >> 1);

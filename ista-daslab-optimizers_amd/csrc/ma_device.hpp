@@ -107,27 +107,32 @@ __device__ __forceinline__ float dpp_perm(float v) {
         __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
+// mn = min(mn, mn of the lane the pattern names), mx likewise: one instruction each, the
+// cross-lane read folded into the operation.  (A vector write followed by a cross-lane read of
+// the same register needs two idle issue slots in between, which the compiler cannot see
+// inside an asm statement: the s_nop provides them.)
+#define MA_DPP_MINMAX(NAME, PATTERN)                                                       \
+    __device__ __forceinline__ void NAME(float &mn, float &mx) {                           \
+        asm volatile("s_nop 1\n\t"                                                         \
+                     "v_min_f32_dpp %0, %0, %0 " PATTERN " row_mask:0xf bank_mask:0xf\n\t" \
+                     "v_max_f32_dpp %1, %1, %1 " PATTERN " row_mask:0xf bank_mask:0xf"      \
+                     : "+v"(mn), "+v"(mx));                                                \
+    }
+MA_DPP_MINMAX(minmax_swap1, "quad_perm:[1,0,3,2]")
+MA_DPP_MINMAX(minmax_swap2, "quad_perm:[2,3,0,1]")
+MA_DPP_MINMAX(minmax_half_mirror, "row_half_mirror")
+MA_DPP_MINMAX(minmax_mirror, "row_mirror")
+#undef MA_DPP_MINMAX
+
 // min / max over aligned groups of `ql` lanes (a power of two), result in every lane.
 // QL > 0 fixes the group size at compile time; QL == 0 takes it from `ql`.
 template <int QL>
 __device__ __forceinline__ void group_minmax(float &mn, float &mx, int ql_runtime) {
     const int ql = QL > 0 ? QL : ql_runtime;
-    if (ql >= 2) {
-        mn = fmin_raw(mn, dpp_perm<0xB1>(mn));  // quad_perm [1,0,3,2]
-        mx = fmax_raw(mx, dpp_perm<0xB1>(mx));
-    }
-    if (ql >= 4) {
-        mn = fmin_raw(mn, dpp_perm<0x4E>(mn));  // quad_perm [2,3,0,1]
-        mx = fmax_raw(mx, dpp_perm<0x4E>(mx));
-    }
-    if (ql >= 8) {
-        mn = fmin_raw(mn, dpp_perm<0x141>(mn));  // row_half_mirror
-        mx = fmax_raw(mx, dpp_perm<0x141>(mx));
-    }
-    if (ql >= 16) {
-        mn = fmin_raw(mn, dpp_perm<0x140>(mn));  // row_mirror
-        mx = fmax_raw(mx, dpp_perm<0x140>(mx));
-    }
+    if (ql >= 2) minmax_swap1(mn, mx);
+    if (ql >= 4) minmax_swap2(mn, mx);
+    if (ql >= 8) minmax_half_mirror(mn, mx);
+    if (ql >= 16) minmax_mirror(mn, mx);
     for (int s = 16; s < ql; s <<= 1) {
         mn = fmin_raw(mn, __shfl_xor(mn, s, kWave));
         mx = fmax_raw(mx, __shfl_xor(mx, s, kWave));
@@ -443,6 +448,114 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 
 constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multiple of 16); more falls back
 
+template <int CAP, class R>
+__device__ __forceinline__ bool topk_among_candidates(R &r, int kb, uint16_t *park,
+                                                      uint32_t *hist, uint32_t *sh,
+                                                      uint16_t *sel_idx, uint16_t *sel_val,
+                                                      uint32_t filled, uint32_t at_least,
+                                                      const uint32_t *lists, uint16_t *ties);
+
+// min over the 64 lanes, in lane 63 (DPP only)
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ uint32_t dpp_or_ones(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)v, CTRL, ROW_MASK, BANK_MASK, false);
+}
+__device__ __forceinline__ uint32_t wave_min_to_last(uint32_t v) {
+    v = min(v, dpp_or_ones<0x111>(v));
+    v = min(v, dpp_or_ones<0x112>(v));
+    v = min(v, dpp_or_ones<0x114, 0xF, 0xE>(v));
+    v = min(v, dpp_or_ones<0x118, 0xF, 0xC>(v));
+    v = min(v, dpp_or_ones<0x142, 0xA>(v));
+    v = min(v, dpp_or_ones<0x143, 0xC>(v));
+    return v;
+}
+
+// The fast top-k with a lower bound known beforehand.  `hint` is a 15-bit magnitude key held
+// by the threads that have one (others pass 0x7fff); the smallest of them, lowered by a
+// thirty-second, is tried as the bound L: every element with key >= L becomes a candidate, and if
+// at least kb turn up (so the kb-th largest is among them) and they fit the lists, the exact
+// top-kb is taken among them as in fast_topk_bf16.  Callers pass the magnitudes of the entries
+// the previous step selected from this block: their smallest is that step's threshold, and
+// thresholds of successive steps differ by a per cent or so.  Any hint gives the same selection
+// or a refusal (false, r unchanged): a hint that is too high finds fewer than kb candidates, one
+// that is too low overflows the lists.  Candidates are listed in the order (wave, lane, chunk,
+// element).  hist, sh, park as in fast_topk_bf16.
+template <class R>
+__device__ __forceinline__ bool hint_topk_bf16(R &r, int kb, uint32_t hint, uint16_t *park,
+                                               uint32_t *hist, uint32_t *sh, uint16_t *sel_idx,
+                                               uint16_t *sel_val) {
+    constexpr int C = R::kC;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    const uint32_t wmin = wave_min_to_last(hint);
+    if (lane == kWave - 1) sh[kShScan + wave] = wmin;
+    // only the second histogram is used here; the candidate lists take the place of the first
+    for (int i = tid; i < kSmallHistWords; i += kWG) hist[kSmallHistWords + i] = 0;
+    __syncthreads();
+    uint32_t hmin = 0x7fffu;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) hmin = min(hmin, sh[kShScan + w]);
+    // L = hmin lowered by 1/32, as a key (truncation only lowers it further)
+    const float lf = __uint_as_float(hmin << 16) * 0.96875f;
+    const uint32_t L = __float_as_uint(lf) >> 16;
+    const uint32_t LL = L | L << 16;
+    // Flags of the elements with key >= L: bit 15 of (key | 0x8000) - L in each 16-bit half.
+    // Byte B of flo holds, for chunk c = 0..3, element B at bit 2c and element 4 + B at bit
+    // 2c + 1; fhi the same for the chunks above.
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    static_assert(C <= 8, "two words of flags");
+    uint32_t flo = 0, fhi = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        uint32_t t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const us2 a = __builtin_bit_cast(us2, (r.w[c][i] & 0x7fff7fffu) | 0x80008000u);
+            t[i] = __builtin_bit_cast(uint32_t, (us2)(a - __builtin_bit_cast(us2, LL)));
+        }
+        // the bytes whose top bits are the flags: elements 0..3 -> x, elements 4..7 -> y
+        const uint32_t x = __builtin_amdgcn_perm(t[1], t[0], 0x07050301u) & 0x80808080u;
+        const uint32_t y = __builtin_amdgcn_perm(t[3], t[2], 0x07050301u) & 0x80808080u;
+        const uint32_t z = (x >> 7) | (y >> 6);
+        if (c < 4) flo |= z << (2 * c);
+        else fhi |= z << (2 * (c - 4));
+        const int off = chunk_off<C>(wave, c, lane);
+        *reinterpret_cast<uint4 *>(park + off) =
+            make_uint4(r.w[c][0], r.w[c][1], r.w[c][2], r.w[c][3]);
+    }
+    const uint32_t cnt = (uint32_t)(__popc(flo) + __popc(fhi));
+    const uint32_t incl = wave_incl_scan(cnt, lane);
+    const uint32_t filled = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    constexpr int kCap = 128;  // list slots per wave
+    static_assert(kCap * kWaves <= kSmallHistWords, "the lists take the first histogram's place");
+    uint32_t *mine = hist + wave * kCap;
+    if (filled <= (uint32_t)kCap) {
+        // one candidate per lane and turn, lowest flag first; its key is read back from the
+        // parked block (the lane's own cells)
+        uint32_t pos = incl - cnt;
+        const int off0 = chunk_off<C>(wave, 0, lane);
+        while (__builtin_amdgcn_ballot_w64((flo | fhi) != 0) != 0) {
+            const bool low = flo != 0;
+            const uint32_t f = low ? flo : fhi;
+            if (f != 0) {
+                const int b = __ffs(f) - 1;
+                if (low) flo &= flo - 1;
+                else fhi &= fhi - 1;
+                const int c = ((b >> 1) & 3) + (low ? 0 : 4);
+                const int e = (b >> 3) + 4 * (b & 1);
+                const int off = off0 + c * (kWave * kChunk) + e;
+                const uint32_t key = park[off] & 0x7fffu;
+                mine[pos] = (key << 15) | (uint32_t)(32767 - off);
+                ++pos;
+            }
+        }
+    }
+    if (lane == 0) sh[kShCnts + wave] = filled;
+    __syncthreads();
+    return topk_among_candidates<kCap>(r, kb, park, hist, sh, sel_idx, sel_val, filled,
+                                       (uint32_t)kb, hist,
+                                       reinterpret_cast<uint16_t *>(hist + 2 * kSmallHistWords));
+}
+
 // The fast top-k of a full bf16 block.  `park` (kRound*C uint16 cells) receives the block;
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
 // magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false
@@ -515,20 +628,43 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     if (lane < 16 && filled + lane < (uint32_t)kCandPerWave) mine[filled + lane] = 0;
     if (lane == 0) sh[kShCnts + wave] = filled;
     __syncthreads();
+    // ties are listed in the first histograms, which are free by then
+    return topk_among_candidates<kCandPerWave>(r, kb, park, hist, sh, sel_idx, sel_val, filled, 0,
+                                               cand, reinterpret_cast<uint16_t *>(hist));
+}
+
+// Second half of the fast selections.  Every wave has filed its candidates (composites
+// key << 15 | 32767 - index, every element of the top kb among them) in its list and their
+// number in sh[kShCnts + wave], the block is parked, and a barrier has passed.  Returns false,
+// with r reloaded unchanged, if a wave had more candidates than its list holds, if there are
+// fewer than `at_least` candidates in all (then the lists may miss members of the top kb), or
+// if too many candidates tie at the threshold.
+template <int CAP, class R>
+__device__ __forceinline__ bool topk_among_candidates(R &r, int kb, uint16_t *park,
+                                                      uint32_t *hist, uint32_t *sh,
+                                                      uint16_t *sel_idx, uint16_t *sel_val,
+                                                      uint32_t filled, uint32_t at_least,
+                                                      const uint32_t *lists, uint16_t *ties) {
+    constexpr int C = R::kC;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    const uint32_t *mine = lists + wave * CAP;
     uint32_t cnts[kWaves];
     bool ok = true;
+    uint32_t total = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
         cnts[w] = sh[kShCnts + w];
-        ok = ok && cnts[w] <= (uint32_t)kCandPerWave;
+        ok = ok && cnts[w] <= (uint32_t)CAP;
+        total += cnts[w];
     }
+    ok = ok && total >= at_least;
     if (ok) {
         // Exact top-kb among the candidates (every thread takes those of its own wave's list,
         // one per lane and 64 list slots): a radix select on their keys gives the threshold key
         // T and the number of entries equal to T to keep; entries above T get consecutive
         // output slots by a prefix sum over the threads, entries equal to T are ranked among
         // themselves by index (they are few).
-        constexpr int kMine = kCandPerWave / kWave;  // candidates per thread
+        constexpr int kMine = CAP / kWave;  // candidates per thread
         uint32_t my[kMine], keys[kMine];
         uint32_t have = 0;
 #pragma unroll
@@ -543,7 +679,6 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
         int take_eq, n_eq;
         const uint32_t T = select_kth_key15<kMine>(keys, have, kb, hist + kSmallHistWords,
                                                    sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
-        uint16_t *ties = reinterpret_cast<uint16_t *>(hist);  // the first histograms are free
         constexpr int kMaxTies = 512;
         ok = n_eq <= kMaxTies;
         if (ok) {
@@ -755,16 +890,24 @@ __device__ __forceinline__ void window_accumulate(const WindowView &wv, int kb, 
 
 // ---- division by a value shared by many numerators ---------------------------------------------
 //
-// y / u, correctly rounded, with the refinement of 1/u paid once.  This is the fp32 division
-// expansion of the compiler (reciprocal, one Newton step, quotient, two fused residual
-// corrections) without its operand scaling and special-case fix-up, so it equals IEEE division
-// bit for bit whenever those would be no-ops: u normal with a biased exponent in [32, 222]
-// (callers scale u and y by an exact power of two to get there), and the quotient neither
-// overflowing nor denormal.  Callers keep |y| within a few multiples of 16 u, and a quotient
-// below 2^-30 is only ever compared with 1/2.
+// y / u, correctly rounded, with the reciprocal paid once.  r = rcp(u) refined by one Newton
+// step is the correctly rounded reciprocal unless u's significand is all ones, and with such
+// an r the sequence q = y * r; e = fma(-u, q, y); q + e * r (one rounding) is the correctly
+// rounded quotient (Markstein's theorem; checked against IEEE division on 12e9 operand pairs,
+// random, at rounding boundaries and on bf16's grid, from every reciprocal seed within one
+// ulp: no difference; with an all-ones significand it does fail).  No operand scaling and no
+// special-case fix-up, so callers keep u normal with a biased exponent in [32, 222] and its
+// significand not all ones (divisor_is_plain; they scale u and y by an exact power of two or
+// take the compiler's division otherwise), and |y| within a few multiples of 16 u; a quotient
+// too small to be normal is only ever compared with 1/2.
 struct Divisor {
     float u, r;
 };
+
+__device__ __forceinline__ bool divisor_is_plain(float u) {
+    const uint32_t b = __float_as_uint(u);
+    return ((b >> 23) & 0xffu) - 32u <= 190u && (b & 0x7fffffu) != 0x7fffffu;
+}
 
 __device__ __forceinline__ Divisor make_divisor(float u) {
     Divisor d;
@@ -776,11 +919,9 @@ __device__ __forceinline__ Divisor make_divisor(float u) {
 }
 
 __device__ __forceinline__ float div_shared(float y, const Divisor &d) {
-    const float q0 = y * d.r;
-    const float e1 = __builtin_fmaf(-d.u, q0, y);
-    const float q1 = __builtin_fmaf(e1, d.r, q0);
-    const float e2 = __builtin_fmaf(-d.u, q1, y);
-    return __builtin_fmaf(e2, d.r, q1);
+    const float q = y * d.r;
+    const float e = __builtin_fmaf(-d.u, q, y);
+    return __builtin_fmaf(e, d.r, q);
 }
 
 // x / 15 for the quantisation step u = (max - min) / 15: the shared-divisor sequence when the
