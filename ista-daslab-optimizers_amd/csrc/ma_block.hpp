@@ -459,7 +459,10 @@ struct FusedBlock {
             const float mn = bf2f(mnb), mx = bf2f(mxb);
             const float u = div15(mx - mn, d15);
             // the nibbles as bytes of two words (even elements high), one conversion each
-            const uint32_t odd = cw[c] & 0x0f0f0f0fu, even = (cw[c] >> 4) & 0x0f0f0f0fu;
+            uint32_t odd = cw[c] & 0x0f0f0f0fu, even = (cw[c] >> 4) & 0x0f0f0f0fu;
+            // (hidden from the optimiser, which would turn the byte reads back into bit-field
+            // extracts of cw, one more instruction per element)
+            asm volatile("" : "+v"(odd), "+v"(even));
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
                 const uint32_t code = (((e & 1) ? odd : even) >> (8 * (e >> 1))) & 0xffu;
@@ -654,9 +657,14 @@ struct FusedBlock {
         constexpr int kSlots = 5;  // four entries of an older row, one of this step's row
         const TensorDesc &D = G.D;
         const int kb = G.kb;
-        uint32_t *lcount = sh + kShLinks;
-        const int cap = (P.L.total - P.L.off_union) / 8;
-        float *f1 = reinterpret_cast<float *>(hist), *f2 = f1 + cap;
+        // entries of coordinates that several rows name wait in a queue: key, two terms and a
+        // link cell each, at most one per thread
+        uint32_t *lcount = sh + kShLinks, *qcount = sh + kShCounter;
+        constexpr int kQueue = kWG;
+        uint32_t *qkey = hist;
+        float *qa1 = reinterpret_cast<float *>(hist + kQueue), *qa2 = qa1 + kQueue;
+        uint16_t *link = reinterpret_cast<uint16_t *>(qa2 + kQueue);
+        const bool queue_fits = P.L.total - P.L.off_union >= kQueue * 14;
         if (!slot_clear) {
             __syncthreads();  // the LDS of the selection is reused below
             for (int i = tid; i < n / 8; i += kWG)
@@ -666,7 +674,7 @@ struct FusedBlock {
             sh[kShW1 + tid] = __float_as_uint(P.W.w1[tid]);
             sh[kShW2 + tid] = __float_as_uint(P.W.w2[tid]);
         }
-        if (tid == 0) *lcount = 0;
+        if (tid == 0) *lcount = *qcount = 0;
         __syncthreads();
         // ---- every entry marks its row in the cell of its coordinate
         uint32_t tag[kSlots];  // index | value << 16; all ones: no entry
@@ -692,103 +700,106 @@ struct FusedBlock {
             if (have) atomicOr(cell32 + (idx >> 1), (1u << myrow[j]) << ((idx & 1u) * 16));
         }
         __syncthreads();
-        // ---- a coordinate named by one row has its sums from that entry; the lowest row of
-        //      the others reserves the coordinate's list
+        // ---- a coordinate named by one row has its sums from that entry; the entries of the
+        //      others queue up with their rank among the coordinate's rows
         const float w1_old = w_row >= 0 ? __uint_as_float(sh[kShW1 + w_row]) : 0.0f;
         const float w2_old = w_row >= 0 ? __uint_as_float(sh[kShW2 + w_row]) : 0.0f;
         const float w1_cur = __uint_as_float(sh[kShW1 + D.row]);
         const float w2_cur = __uint_as_float(sh[kShW2 + D.row]);
-        float z1[kSlots], z2[kSlots];  // the entry's terms, then (owners) the coordinate's sums
-        uint32_t aux[kSlots];  // 0: the coordinate is this entry's alone; else its rows (mask)
-                               // and, for the lowest of them, the list's first cell << 16
-        uint32_t owner = 0;    // bit j: slot j computes the update of its coordinate
+        constexpr int kOwned = kSlots + 1;  // the last: a queued coordinate this thread sums
+        float z1[kOwned], z2[kOwned];       // sums of the coordinates this thread updates
+        uint32_t own[kOwned];               // their indices; all ones: none
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) {
-            aux[j] = 0;
+            own[j] = 0xffffffffu;
             z1[j] = z2[j] = 0.0f;
             if (tag[j] != 0xffffffffu) {
                 const uint32_t idx = tag[j] & 0xffffu, row = (uint32_t)myrow[j];
                 const uint32_t mask = cell16[idx];
                 const float v = bf2f(tag[j] >> 16);
                 const float vv = v * v;
-                z1[j] = (j < 4 ? w1_old : w1_cur) * v;
-                z2[j] = (j < 4 ? w2_old : w2_cur) * vv;
+                const float a1 = (j < 4 ? w1_old : w1_cur) * v;
+                const float a2 = (j < 4 ? w2_old : w2_cur) * vv;
                 if (mask == 1u << row) {
-                    z1[j] = 0.0f + z1[j];
-                    z2[j] = 0.0f + z2[j];
-                    owner |= 1u << j;
+                    z1[j] = 0.0f + a1;
+                    z2[j] = 0.0f + a2;
+                    own[j] = idx;
                 } else {
-                    aux[j] = mask;
-                    if ((mask & ((1u << row) - 1u)) == 0) {
-                        aux[j] |= atomicAdd(lcount, (uint32_t)__popc(mask)) << 16;
-                        owner |= 1u << j;
+                    const uint32_t at = atomicAdd(qcount, 1u);
+                    if (at < (uint32_t)kQueue) {
+                        const uint32_t rank = (uint32_t)__popc(mask & ((1u << row) - 1u));
+                        qkey[at] = idx | rank << 15 | (uint32_t)__popc(mask) << 19;
+                        qa1[at] = a1;
+                        qa2[at] = a2;
                     }
                 }
             }
         }
+        own[kSlots] = 0xffffffffu;
+        z1[kSlots] = z2[kSlots] = 0.0f;
         __syncthreads();
-        const uint32_t listed = *lcount;
-        if (listed > (uint32_t)cap) {
-            // more shared coordinates than the lists hold: the general stage, which takes its
-            // entries in its own order and serves shared coordinates row by row
+        const uint32_t queued = *qcount;
+        if (queued > (uint32_t)kQueue || !queue_fits) {
+            // more entries share coordinates than the queue holds: the general stage, which
+            // takes its entries in its own order and serves shared coordinates row by row
             slot_clear = false;
             load_window(G);
             window_stage(G);
             param_stage(G);
             return;
         }
-        if (listed != 0) {
-#pragma unroll
-            for (int j = 0; j < kSlots; ++j)
-                if (aux[j] != 0 && ((owner >> j) & 1u) != 0)
-                    cell16[tag[j] & 0xffffu] = (uint16_t)(aux[j] >> 16);
-            __syncthreads();
-#pragma unroll
-            for (int j = 0; j < kSlots; ++j) {
-                if (aux[j] != 0) {
-                    const uint32_t mask = aux[j] & 0xffffu;
-                    const uint32_t at = (uint32_t)cell16[tag[j] & 0xffffu] +
-                                        (uint32_t)__popc(mask & ((1u << myrow[j]) - 1u));
-                    if (at < (uint32_t)cap) {
-                        f1[at] = z1[j];
-                        f2[at] = z2[j];
-                    }
-                }
+        if (queued != 0) {
+            // queued entry t belongs to thread t.  The lowest row of a coordinate reserves one
+            // link cell per row and leaves the first cell's number in the coordinate's cell
+            // (the marks are not needed any more); every entry files its queue position at its
+            // rank; the lowest row adds the terms in that order, the order of the rows.
+            uint32_t key = 0;
+            const bool mine = (uint32_t)tid < queued;
+            if (mine) {
+                key = qkey[tid];
+                if (((key >> 15) & 15u) == 0)
+                    cell16[key & 0x7fffu] = (uint16_t)atomicAdd(lcount, key >> 19);
             }
             __syncthreads();
-#pragma unroll
-            for (int j = 0; j < kSlots; ++j) {
-                if (aux[j] != 0 && ((owner >> j) & 1u) != 0) {
-                    const uint32_t base = aux[j] >> 16;
-                    const int terms = __popc(aux[j] & 0xffffu);
-                    float s1 = 0.0f, s2 = 0.0f;
-                    for (int r = 0; r < terms; ++r) {
-                        uint32_t at = base + (uint32_t)r;
-                        at = at < (uint32_t)cap ? at : (uint32_t)cap - 1u;
-                        s1 = s1 + f1[at];
-                        s2 = s2 + f2[at];
-                    }
-                    z1[j] = s1;
-                    z2[j] = s2;
+            uint32_t base = 0;
+            if (mine) {
+                base = cell16[key & 0x7fffu];  // the cells are not read again after this
+                uint32_t at = base + ((key >> 15) & 15u);
+                at = at < (uint32_t)kQueue ? at : (uint32_t)kQueue - 1u;
+                link[at] = (uint16_t)tid;
+            }
+            __syncthreads();
+            if (mine && ((key >> 15) & 15u) == 0) {
+                const int terms = (int)(key >> 19);
+                float s1 = 0.0f, s2 = 0.0f;
+                for (int r = 0; r < terms; ++r) {
+                    uint32_t at = base + (uint32_t)r;
+                    at = at < (uint32_t)kQueue ? at : (uint32_t)kQueue - 1u;
+                    uint32_t q = link[at];
+                    q = q < (uint32_t)kQueue ? q : (uint32_t)kQueue - 1u;
+                    s1 = s1 + qa1[q];
+                    s2 = s2 + qa2[q];
                 }
+                z1[kSlots] = s1;
+                z2[kSlots] = s2;
+                own[kSlots] = key & 0x7fffu;
             }
         }
-        uint32_t upd[kSlots];  // index | update's bf16 bits << 16; all ones: none
+        uint32_t upd[kOwned];  // index | update's bf16 bits << 16; all ones: none
 #pragma unroll
-        for (int j = 0; j < kSlots; ++j) {
+        for (int j = 0; j < kOwned; ++j) {
             upd[j] = 0xffffffffu;
-            if (((owner >> j) & 1u) != 0) {
+            if (own[j] != 0xffffffffu) {
                 const float u = adam_direction(z1[j], z2[j], P.W.s1, P.W.s2, P.W.eps);
-                upd[j] = (tag[j] & 0xffffu) | f2bf(u) << 16;
+                upd[j] = own[j] | f2bf(u) << 16;
             }
         }
-        // nobody reads the cells' marks any more (the last readers passed a barrier above, or
-        // there were no lists)
+        // nobody reads the cells' marks any more: the last readers passed a barrier above
         const float neg_lr = D.neg_lr;
         if (D.apply_decay != 0) {
             // every parameter changes: the updates go to the cells, the dense stage does the rest
 #pragma unroll
-            for (int j = 0; j < kSlots; ++j)
+            for (int j = 0; j < kOwned; ++j)
                 if (upd[j] != 0xffffffffu) cell16[upd[j] & 0xffffu] = (uint16_t)(upd[j] >> 16);
             __syncthreads();
             param_stage(G);
@@ -799,7 +810,7 @@ struct FusedBlock {
             *reinterpret_cast<uint4 *>(cell16 + chunk_off<C>(wave, c, lane)) = praw[c].q;
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < kSlots; ++j) {
+        for (int j = 0; j < kOwned; ++j) {
             if (upd[j] != 0xffffffffu) {
                 const uint32_t idx = upd[j] & 0xffffu;
                 const float prod = neg_lr * bf2f(upd[j] >> 16);
@@ -1725,10 +1736,10 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
             fb.window_stage(G);
             fb.param_stage_dense(G);
         } else {
-            fb.quantize(G);
-            // asked for only now: measured faster than at the start of the block, where they
-            // keep 30 more registers live through the selection and the quantisation
+            // parameters and window entries are asked for before the quantisation, which
+            // hides their latency (the selection runs with more registers free without them)
             fb.load_params_window(G);
+            fb.quantize(G);
             if constexpr (HOLD) fb.load_held(G, true);
             fb.update(G);
         }

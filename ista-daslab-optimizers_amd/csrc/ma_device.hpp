@@ -446,6 +446,54 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
     return prefix;
 }
 
+// The same selection in one pass for keys known to be at least `base`: the digit is
+// min(key - base, 255), so every bin below 255 is one key value.  Returns the kb-th largest key
+// as select_kth_key15 does, or 0xffffffff if it fell into the bin of the keys base + 255 and
+// above (then nothing else is valid either).  hist: 257 * kSmallCopies zero words; shp: 2 words.
+template <int N>
+__device__ __forceinline__ uint32_t select_kth_near(const uint32_t (&v)[N], uint32_t valid,
+                                                    int kb, uint32_t base, uint32_t *hist,
+                                                    uint32_t *shp, uint32_t *sh_neq,
+                                                    int &take_eq, int &n_eq) {
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const uint32_t off = v[i] - base;
+        const uint32_t bin = ((valid >> i) & 1u) != 0 ? (off < 255u ? off : 255u) : 256u;
+        atomicAdd(&hist[bin * kSmallCopies + (lane & (kSmallCopies - 1))], 1u);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        uint32_t c[4], tot = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int bin = 255 - 4 * lane - i;
+            c[i] = 0;
+#pragma unroll
+            for (int k = 0; k < kSmallCopies; ++k) c[i] += hist[bin * kSmallCopies + k];
+            tot += c[i];
+        }
+        const uint32_t incl = wave_incl_scan(tot, lane);
+        uint32_t above = incl - tot;
+        if (above < (uint32_t)kb && (uint32_t)kb <= incl) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (above < (uint32_t)kb && (uint32_t)kb <= above + c[i]) {
+                    shp[0] = (uint32_t)(255 - 4 * lane - i);
+                    shp[1] = (uint32_t)kb - above;
+                    *sh_neq = c[i];
+                }
+                above += c[i];
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t bin = shp[0];
+    take_eq = (int)shp[1];
+    n_eq = (int)*sh_neq;
+    return bin < 255u ? base + bin : 0xffffffffu;
+}
+
 constexpr int kCandPerWave = 512 / kWaves;  // candidate slots per wave (a multiple of 16); more falls back
 
 template <int CAP, class R>
@@ -453,7 +501,8 @@ __device__ __forceinline__ bool topk_among_candidates(R &r, int kb, uint16_t *pa
                                                       uint32_t *hist, uint32_t *sh,
                                                       uint16_t *sel_idx, uint16_t *sel_val,
                                                       uint32_t filled, uint32_t at_least,
-                                                      const uint32_t *lists, uint16_t *ties);
+                                                      const uint32_t *lists, uint16_t *ties,
+                                                      uint32_t key_base);
 
 // min over the 64 lanes, in lane 63 (DPP only)
 template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
@@ -553,7 +602,8 @@ __device__ __forceinline__ bool hint_topk_bf16(R &r, int kb, uint32_t hint, uint
     __syncthreads();
     return topk_among_candidates<kCap>(r, kb, park, hist, sh, sel_idx, sel_val, filled,
                                        (uint32_t)kb, hist,
-                                       reinterpret_cast<uint16_t *>(hist + 2 * kSmallHistWords));
+                                       reinterpret_cast<uint16_t *>(hist + 2 * kSmallHistWords),
+                                       L);
 }
 
 // The fast top-k of a full bf16 block.  `park` (kRound*C uint16 cells) receives the block;
@@ -630,7 +680,7 @@ __device__ __forceinline__ bool fast_topk_bf16(R &r, int kb, uint16_t *park, uin
     __syncthreads();
     // ties are listed in the first histograms, which are free by then
     return topk_among_candidates<kCandPerWave>(r, kb, park, hist, sh, sel_idx, sel_val, filled, 0,
-                                               cand, reinterpret_cast<uint16_t *>(hist));
+                                               cand, reinterpret_cast<uint16_t *>(hist), 0);
 }
 
 // Second half of the fast selections.  Every wave has filed its candidates (composites
@@ -644,7 +694,8 @@ __device__ __forceinline__ bool topk_among_candidates(R &r, int kb, uint16_t *pa
                                                       uint32_t *hist, uint32_t *sh,
                                                       uint16_t *sel_idx, uint16_t *sel_val,
                                                       uint32_t filled, uint32_t at_least,
-                                                      const uint32_t *lists, uint16_t *ties) {
+                                                      const uint32_t *lists, uint16_t *ties,
+                                                      uint32_t key_base) {
     constexpr int C = R::kC;
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     const uint32_t *mine = lists + wave * CAP;
@@ -677,10 +728,16 @@ __device__ __forceinline__ bool topk_among_candidates(R &r, int kb, uint16_t *pa
         }
         if (tid == 0) sh[kShTies] = 0;
         int take_eq, n_eq;
-        const uint32_t T = select_kth_key15<kMine>(keys, have, kb, hist + kSmallHistWords,
-                                                   sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
+        // candidates known to lie at or above a key (the hinted selection's bound; at least
+        // kb of them, so the kb-th exists) are told apart in one pass
+        const uint32_t T =
+            key_base != 0
+                ? select_kth_near<kMine>(keys, have, kb, key_base, hist + kSmallHistWords,
+                                         sh + kShSel + 4, sh + kShNEq, take_eq, n_eq)
+                : select_kth_key15<kMine>(keys, have, kb, hist + kSmallHistWords,
+                                          sh + kShSel + 4, sh + kShNEq, take_eq, n_eq);
         constexpr int kMaxTies = 512;
-        ok = n_eq <= kMaxTies;
+        ok = n_eq <= kMaxTies && T != 0xffffffffu;
         if (ok) {
             uint32_t n_gt = 0;
 #pragma unroll
