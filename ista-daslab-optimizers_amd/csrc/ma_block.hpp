@@ -8,6 +8,12 @@
 
 namespace ma {
 
+#ifdef MA_EXP_NOSCHED
+#define MA_SCHED_BARRIER() do {} while (0)
+#else
+#define MA_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0)
+#endif
+
 
 // LDS map shared by the block kernels (byte offsets from the start of dynamic LDS)
 struct LdsMap {
@@ -441,23 +447,28 @@ struct FusedBlock {
     // ---- a = g + Qinv(e), rounded to the element type (MA:190)
     __device__ __forceinline__ void dequant(const BlockGeo &G) {
         const int n = FULL ? C * kRound : G.n;
+        // with the wave's statistics spread over the lanes, each lane forms the step of the
+        // quantisation blocks it holds once, and the chunks fetch (min, step)
+        float su[kCoStats];
+        if constexpr (kCoop) {
+#pragma unroll
+            for (int i = 0; i < kCoStats; ++i) su[i] = div15(bf2f(smx[i]) - bf2f(smn[i]), d15);
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
             float v[8];
             graw[c].to_float(v);
-            uint32_t mnb, mxb;
+            float mn, u;
             if constexpr (kCoop) {
                 const int j0 = c * (kWave / QL);  // first statistic of this chunk in the wave
                 const int src = (j0 & (kWave - 1)) + lane / QL;
-                mnb = (uint32_t)__shfl((int)smn[j0 >> 6], src, kWave);
-                mxb = (uint32_t)__shfl((int)smx[j0 >> 6], src, kWave);
+                mn = bf2f((uint32_t)__shfl((int)smn[j0 >> 6], src, kWave));
+                u = __int_as_float(__shfl(__float_as_int(su[j0 >> 6]), src, kWave));
             } else {
-                mnb = smn[c];
-                mxb = smx[c];
+                mn = bf2f(smn[c]);
+                u = div15(bf2f(smx[c]) - mn, d15);
             }
-            const float mn = bf2f(mnb), mx = bf2f(mxb);
-            const float u = div15(mx - mn, d15);
             // the nibbles as bytes of two words (even elements high), one conversion each
             uint32_t odd = cw[c] & 0x0f0f0f0fu, even = (cw[c] >> 4) & 0x0f0f0f0fu;
             // (hidden from the optimiser, which would turn the byte reads back into bit-field
@@ -476,7 +487,7 @@ struct FusedBlock {
                     if (off + e >= n) v[e] = 0.0f;
             }
             r.set_chunk(c, v);
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
         launder(r);
     }
@@ -556,7 +567,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
     }
 
@@ -1164,7 +1175,7 @@ struct FusedBlock {
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
     }
 
@@ -1243,7 +1254,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
     }
 
@@ -1279,7 +1290,7 @@ struct FusedBlock {
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
     }
 
@@ -1518,7 +1529,7 @@ struct FusedBlock {
                     if (off + e >= n) v[e] = 0.0f;
             }
             r.set_chunk(c, v);
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
         launder(r);
     }
@@ -1661,7 +1672,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            MA_SCHED_BARRIER();
         }
         span_store_statistics(G, S);
     }
@@ -1705,6 +1716,9 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     auto run = [&](auto &fb) {
         fb.load_grad_inputs(G);
         fb.dequant(G);
+#ifdef MA_EXP_EARLY3
+        if constexpr (!DENSE) fb.load_params_window(G);
+#endif
         // the older window rows are most of this path's traffic: asked for before the selection
         if constexpr (HOLD) fb.load_held(G, false);
 #ifdef MA_EXP_SKIP_TOPK
@@ -1738,7 +1752,9 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         } else {
             // parameters and window entries are asked for before the quantisation, which
             // hides their latency (the selection runs with more registers free without them)
+#ifndef MA_EXP_EARLY3
             fb.load_params_window(G);
+#endif
             fb.quantize(G);
             if constexpr (HOLD) fb.load_held(G, true);
             fb.update(G);

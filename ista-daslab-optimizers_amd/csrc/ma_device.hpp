@@ -989,12 +989,31 @@ __device__ __forceinline__ float div15(float x, const Divisor &d15) {
     return x / 15.0f;
 }
 
+// (z1 s1) / (eps + sqrt(z2 s2)), square root and quotient correctly rounded.
+// Short way: the square root by Goldschmidt's iteration from rsq (g = x y, h = y / 2 refined
+// once together, then g + (x - g g) h in one rounding: equal to the correctly rounded root for
+// every significand and every seed within two ulp of 1 / sqrt(x), checked exhaustively), the
+// quotient by div_shared's sequence.  Both without scaling or special cases, so a wave in which
+// some lane's operands are zero, tiny, huge or not finite takes the compiler's expansions.
 __device__ __forceinline__ float adam_direction(float z1, float z2, float s1, float s2,
                                                 float eps) {
     const float mh = z1 * s1;
     const float vh = z2 * s2;
-    const float den = eps + sqrtf(vh);
-    return mh / den;
+    const float y = __builtin_amdgcn_rsqf(vh);
+    float g = vh * y, h = 0.5f * y;
+    const float r = __builtin_fmaf(-h, g, 0.5f);
+    g = __builtin_fmaf(g, r, g);
+    h = __builtin_fmaf(h, r, h);
+    const float d = __builtin_fmaf(-g, g, vh);
+    const float root = __builtin_fmaf(d, h, g);
+    const float den = eps + root;
+    const float u = div_shared(mh, make_divisor(den));
+    // vh in [2^-90, 2^90], |mh| in [2^-40, 2^90], den plain: then nothing above leaves the
+    // normal range and the quotient is normal
+    const uint32_t ev = (__float_as_uint(vh) >> 23) & 0xffu, em = (__float_as_uint(mh) >> 23) & 0xffu;
+    const bool fine = ev - 37u <= 180u && em - 87u <= 130u && divisor_is_plain(den);
+    if (__builtin_amdgcn_ballot_w64(!fine) == 0) return u;
+    return mh / (eps + sqrtf(vh));
 }
 
 }  // namespace ma
