@@ -3,8 +3,8 @@
 A "step" is one `optimizer.step()` over the whole parameter list of the workload, with
 parameters, gradients and optimizer state already resident in HBM.  The default workload is the
 Llama-2-7B-shaped list (6.74 B bf16 parameters, m=10, k=1 %, quant block 64, alpha=0).
-Gradients are synthetic N(0, 1e-3^2) bf16, drawn on the device before the timed region; a few
-distinct gradient sets are rotated so that consecutive steps see different data.
+Gradients are synthetic N(0, 1e-3^2) bf16, drawn on the device before the timed region; m + 2
+distinct gradient sets are used in turn, so that no gradient recurs inside the window.
 
 Prints ONE JSON line: params/s (whole job), ms per step, the HBM roofline of the fused step
 kernel (algorithmic bytes per parameter x parameters / measured duration against 8 TB/s) and a
@@ -82,9 +82,12 @@ def numel(shape):
     return n
 
 
-def algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, d_block_size, steps_done):
+def algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, d_block_size, first_step,
+                                n_steps):
     """Every array of the step touched once: read g, read+write 4-bit EF, read+write p, write
-    one window row (int16 + bf16), read min(t, m) window rows, read+write bf16 min/max."""
+    one window row (int16 + bf16), read min(t, m) window rows, read+write bf16 min/max.
+    Averaged over the timed steps t = first_step .. first_step + n_steps - 1 (a step with a
+    window that is still filling reads fewer rows)."""
     import math
     s = 2 if dtype == "bf16" else 4
     total_d = total_k = total_stats = 0
@@ -96,7 +99,7 @@ def algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, d_block_size
         total_d += d
         total_k += k
         total_stats += (d + q - 1) // q
-    rows = min(steps_done, m)
+    rows = sum(min(t, m) for t in range(first_step, first_step + n_steps)) / n_steps
     b = total_d * (s + 0.5 + 0.5 + 2 * s) + total_k * 4 * (1 + rows) + total_stats * 8
     if alpha > 0:
         b += total_d * 1.0  # the EF is read and written a second time
@@ -409,7 +412,7 @@ def main():
     kernel_ms = sum(dev_ms) / len(dev_ms)
 
     bpp = algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, opt.d_block_size,
-                                      args.warmup + args.steps)
+                                      args.warmup + 1, args.steps)
     achieved = bpp * n_params / (kernel_ms * 1e-3) / 1e9
     out = {
         "metric": "MicroAdam step throughput (params/s) at the Llama-2-7B shape"
@@ -435,8 +438,9 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op))
                      if args.storage is None else None,
-                     # achieved and traffic are both per step (10 launches of the block kernel
-                     # at 7B): algorithmic bytes of a step / device time of a step
+                     # achieved and traffic are both per step (at 7B: 3 launches of the block
+                     # kernel and one for the norm vectors): algorithmic bytes of a step /
+                     # device time of a step
                      "per": "step", "algorithmic_bytes": bpp * n_params,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},

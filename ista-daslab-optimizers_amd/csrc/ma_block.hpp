@@ -8,12 +8,6 @@
 
 namespace ma {
 
-#ifdef MA_EXP_NOSCHED
-#define MA_SCHED_BARRIER() do {} while (0)
-#else
-#define MA_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0)
-#endif
-
 
 // LDS map shared by the block kernels (byte offsets from the start of dynamic LDS)
 struct LdsMap {
@@ -487,7 +481,7 @@ struct FusedBlock {
                     if (off + e >= n) v[e] = 0.0f;
             }
             r.set_chunk(c, v);
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
         launder(r);
     }
@@ -499,10 +493,8 @@ struct FusedBlock {
         if constexpr (FULL && R::kBF16) {
             if (kb <= kWG) {
                 topk_done = hint_topk_bf16(r, kb, hint, cell16, hist, sh, sel_idx, sel_val);
-#ifndef MA_EXP_NOFALLBACK
                 if (!topk_done)
                     topk_done = fast_topk_bf16(r, kb, cell16, hist, sh, sel_idx, sel_val);
-#endif
                 launder(r);
                 // the block was parked in the slot cells and every thread cleared its own
                 slot_clear = topk_done && P.L.slot_cells == C * kRound;
@@ -567,7 +559,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -1175,7 +1167,7 @@ struct FusedBlock {
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -1254,7 +1246,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -1290,7 +1282,7 @@ struct FusedBlock {
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -1529,7 +1521,7 @@ struct FusedBlock {
                     if (off + e >= n) v[e] = 0.0f;
             }
             r.set_chunk(c, v);
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
         launder(r);
     }
@@ -1672,7 +1664,7 @@ struct FusedBlock {
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
             }
-            MA_SCHED_BARRIER();
+            __builtin_amdgcn_sched_barrier(0);
         }
         span_store_statistics(G, S);
     }
@@ -1706,43 +1698,15 @@ __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
 template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
-#ifdef MA_EXP_NOREMAP
-    const int item = (int)blockIdx.x;
-#else
     const int item = xcd_contiguous_item(P.total_items);
-#endif
     const int ti = find_tensor(P, item);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
     auto run = [&](auto &fb) {
         fb.load_grad_inputs(G);
         fb.dequant(G);
-#ifdef MA_EXP_EARLY3
-        if constexpr (!DENSE) fb.load_params_window(G);
-#endif
         // the older window rows are most of this path's traffic: asked for before the selection
         if constexpr (HOLD) fb.load_held(G, false);
-#ifdef MA_EXP_SKIP_TOPK
-        if (threadIdx.x < G.kb) { fb.sel_idx[threadIdx.x] = threadIdx.x; fb.sel_val[threadIdx.x] = 0; }
-        __syncthreads();
-#else
         fb.topk_and_row(G);
-#endif
-#ifdef MA_EXP_SKIP_QUANT
-        launder(fb.r);
-        fb.load_params_window(G);
-        fb.update(G);
-        return;
-#endif
-#ifdef MA_EXP_SKIP_UPDATE
-        fb.quantize(G);
-        return;
-#endif
-#ifdef MA_EXP_SKIP_WINDOW
-        fb.quantize(G);
-        fb.load_params_window(G);
-        fb.param_stage(G);
-        return;
-#endif
         if constexpr (DENSE) {
             fb.quantize_dense(G);
             fb.load_params(G);
@@ -1752,9 +1716,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         } else {
             // parameters and window entries are asked for before the quantisation, which
             // hides their latency (the selection runs with more registers free without them)
-#ifndef MA_EXP_EARLY3
             fb.load_params_window(G);
-#endif
             fb.quantize(G);
             if constexpr (HOLD) fb.load_held(G, true);
             fb.update(G);
@@ -1776,11 +1738,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
 template <class R, int MIN_WAVES, int PASS>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
-#ifdef MA_EXP_NOREMAP
-    const int item = (int)blockIdx.x;
-#else
     const int item = xcd_contiguous_item(P.total_items);
-#endif
     const int ti = find_tensor(P, item);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
     auto run = [&](auto &fb) {

@@ -354,3 +354,56 @@ def test_logging_step_metrics_do_not_depend_on_the_route(q, sizes):
         sf, so = opts[True][0].state[pf], opts[False][0].state[po]
         for key in ("error", "min_vals", "max_vals"):
             assert torch.equal(sf[key], so[key]), key
+
+
+@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_quantisation_rounding_boundaries(oracle, dtype, use_fused):
+    """The 4-bit codes where they are hardest to get right: every quantisation block holds its
+    minimum 0, its maximum M, and for each of the 15 rounding boundaries the value nearest to
+    (k + 1/2) u and its two neighbours (u = (M - 0) / 15 as the kernels form it), with M running
+    through bf16 significands and through binary exponents -120 .. 120, so that steps u that are
+    tiny, ordinary and huge all occur.  The fused kernels divide by a shared reciprocal where the
+    oracle divides; the codes must agree bit for bit all the same.  A second step with a zero
+    gradient dequantises and requantises them."""
+    from ista_daslab_optimizers import MicroAdam
+    q, DB = 64, 4096
+    sig = [1.0, 1.0078125, 1.25, 1.5, 1.9921875, 1.328125, 1.7109375]
+    exps = list(range(-120, 121, 5))
+    gen = torch.Generator().manual_seed(17)
+    blocks = []
+    for e in exps:
+        for s_ in sig:
+            M = torch.tensor(s_ * 2.0 ** e, dtype=torch.float64).to(dtype)
+            u = (M.float() - 0.0) / 15.0
+            vals = [torch.zeros((), dtype=dtype)] + [M] * 8
+            for k in range(15):
+                x = ((k + 0.5) * u.double()).to(dtype)
+                lo = torch.nextafter(x.float(), torch.tensor(0.0)).to(dtype) if dtype == torch.float32 \
+                    else (x.view(torch.int16) - 1).view(torch.bfloat16)
+                hi = torch.nextafter(x.float(), torch.tensor(float("inf"))).to(dtype) if dtype == torch.float32 \
+                    else (x.view(torch.int16) + 1).view(torch.bfloat16)
+                vals += [lo, x, hi]
+            rnd = (torch.rand(q - len(vals), generator=gen).double() * M.double()).to(dtype)
+            blk = torch.cat([torch.stack(vals), rnd])
+            blocks.append(blk[torch.randperm(q, generator=gen)])
+    g0 = torch.cat(blocks)
+    pad = (-g0.numel()) % DB
+    g0 = torch.cat([g0, torch.zeros(pad, dtype=dtype)])
+    assert torch.isfinite(g0.float()).all()
+    d = g0.numel()
+    p0 = (torch.randn(d, generator=gen) * 0.02).to(dtype)
+    oparams = [to_np(p0)]
+    oref = oracle.OracleMicroAdam(oparams, 4, 1e-3, q, 0.001, 0, d_block_size=DB)
+    gp = torch.nn.Parameter(p0.clone().cuda())
+    opt = MicroAdam([gp], m=4, lr=1e-3, quant_block_size=q, k_init=0.001)
+    opt.d_block_size = DB
+    opt.use_fused = use_fused
+    for step, g in enumerate([g0, torch.zeros_like(g0), g0]):
+        gp.grad = g.clone().cuda()
+        opt.step()
+        oref.step([to_np(g)])
+        assert_state_equal(opt.state[gp], oref.state[0], f"step {step + 1}")
+        assert np.array_equal(to_np(gp.data), oparams[0]), f"step {step + 1}: parameters"
+    codes = oracle.unpack_codes(to_np(opt.state[gp]["error"]), d)
+    assert set(np.unique(codes)) == set(range(16))
