@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <mutex>
+#include <vector>
 
 
 namespace ma {
@@ -453,6 +454,11 @@ static int fused_check(const ma_tensor *t, const ma_hyper *h) {
     if (t->d < q) return MA_ERR_NOT_FUSABLE;
     const bool single = t->d <= h->d_block_size;
     if (!single && (g.dbs % q != 0 || g.dbs % 8 != 0)) return MA_ERR_NOT_FUSABLE;
+    // the block kernels' LDS plans (with and without densification) must fit the hardware
+    const int eb = h->dtype == MA_BF16 ? 2 : 4;
+    if (plan_lds((int)g.dbs, (int)g.k_many, h->m, eb, true, true).total > kLdsLimit ||
+        plan_lds((int)g.dbs, (int)g.k_many, h->m, eb, true, false).total > kLdsLimit)
+        return MA_ERR_LDS;
     return 0;
 }
 
@@ -470,6 +476,9 @@ static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
     if ((q + g.dbs - 1) / g.dbs + 1 > kSpanMaxBlocks) return MA_ERR_NOT_FUSABLE;
     const bool single = t->d <= h->d_block_size;
     if (!single && g.dbs % 8 != 0) return MA_ERR_NOT_FUSABLE;
+    if (plan_lds((int)g.dbs, (int)g.k_many, h->m, h->dtype == MA_BF16 ? 2 : 4, true, false).total >
+        kLdsLimit)
+        return MA_ERR_LDS;
     return 0;
 }
 
@@ -668,6 +677,18 @@ int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
     return fused_check(tensor, hyper);
 }
 
+// One planned launch of a step: the kernel's parameters and the register-tile class it runs in.
+struct PlannedLaunch {
+    FusedParams P;
+    int C;
+};
+
+// Short tensors (one block of up to 4096 / 12288 elements) have kernels of their own, so that
+// they do not occupy a workgroup sized for the hardware block; but when a call holds few of
+// them next to longer tensors, a launch of their own costs more than that: up to this many
+// blocks of a smaller class ride along in the call's largest class instead.
+constexpr int64_t kMergeBlocks = 768;
+
 static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream,
                      bool span, double alpha, void *ws, int64_t ws_bytes) {
     const bool dense = !span && alpha > 0.0;
@@ -688,21 +709,44 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     WindowWeights W;
     window_weights(h->t, h->m, h->beta1, h->beta2, h->eps, &W);
     const int elem_bytes = h->dtype == MA_BF16 ? 2 : 4;
-
-    // Work is handed out in launches of at most kTensorsPerLaunch tensors (their descriptors
-    // travel by value), one workgroup per top-k block, grouped by register-tile class so that
-    // short tensors do not run in the largest kernel.
     const int d_block_size =
         (int)(h->d_block_size > MA_MAX_D_BLOCK ? MA_MAX_D_BLOCK : h->d_block_size);
+
+    // ---- which class every tensor runs in
     static const int classes[4] = {kClass0, kClass1, kClass2, kClass3};
+    std::vector<int> cls(n_tensors);
+    int64_t blocks_in[4] = {0, 0, 0, 0};
+    int largest = 0;
+    for (int i = 0; i < n_tensors; ++i) {
+        const Geometry g = geometry(tensors[i].d, h->d_block_size, h->k_init);
+        const int C = chunks_for(g.dbs);
+        int ci = 0;
+        while (classes[ci] != C) ++ci;
+        cls[i] = ci;
+        blocks_in[ci] += g.n_full + (g.tail > 0 ? 1 : 0);
+        if (ci > largest) largest = ci;
+    }
+    for (int i = 0; i < n_tensors; ++i)
+        if (cls[i] < largest && blocks_in[cls[i]] <= kMergeBlocks) cls[i] = largest;
+
+    // ---- all launches are laid out and checked before the first one starts, so that a call
+    //      either steps every tensor or none
+    std::vector<PlannedLaunch> plan;
     for (int ci = 0; ci < 4; ++ci) {
-        const int C = classes[ci];
-        FusedParams P;
+        int in_class = 0;
+        for (int i = 0; i < n_tensors; ++i)
+            if (cls[i] == ci) ++in_class;
+        if (in_class == 0) continue;
+        // the class's tensors are spread evenly over as few launches as hold them (the
+        // descriptors travel by value, kTensorsPerLaunch at most)
+        const int launches = (in_class + kTensorsPerLaunch - 1) / kTensorsPerLaunch;
+        const int per_launch = (in_class + launches - 1) / launches;
         int count = 0;
-        int64_t items = 0;
+        int64_t items = 0, ws_off = 0;
         int dbs_max = 0, kb_max = 0;
-        auto flush = [&]() -> int {
+        auto close = [&]() -> int {
             if (count == 0) return 0;
+            FusedParams &P = plan.back().P;
             P.n_tensors = count;
             P.W = W;
             P.L = plan_lds(dbs_max, kb_max, h->m, elem_bytes, true, !span && !dense);
@@ -712,49 +756,27 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.q_span = span ? (int32_t)h->quant_block_size : 0;
             P.alpha = (float)alpha;
             P.keep = (float)(1.0 - alpha);
-            if (P.L.total > kLdsLimit) return MA_ERR_LDS;
-            int rc = 0;
-            if (dense) {
-                rc = h->dtype == MA_BF16
-                         ? launch_fused_dense_bf16(C, (unsigned)items, P.L.total, s, P)
-                         : launch_fused_dense_f32(C, (unsigned)items, P.L.total, s, P);
-            } else if (!span) {
-                rc = h->dtype == MA_BF16
-                         ? launch_fused_bf16(C, (unsigned)items, P.L.total, s, P)
-                         : launch_fused_f32(C, (unsigned)items, P.L.total, s, P);
-            } else {
-                const int passes[2] = {alpha > 0.0 ? 1 : 4, alpha > 0.0 ? 2 : 3};
-                for (int i = 0; i < 2 && rc == 0; ++i) {
-                    const int pass = passes[i];
-                    rc = h->dtype == MA_BF16
-                             ? launch_span_bf16(C, pass, (unsigned)items, P.L.total, s, P)
-                             : launch_span_f32(C, pass, (unsigned)items, P.L.total, s, P);
-                }
-            }
             count = 0;
             items = 0;
             dbs_max = kb_max = 0;
-            return rc;
+            return P.L.total > kLdsLimit ? MA_ERR_LDS : 0;
         };
-        // the class's tensors are spread evenly over as few launches as hold them
-        int in_class = 0;
-        for (int i = 0; i < n_tensors; ++i)
-            if (chunks_for(geometry(tensors[i].d, h->d_block_size, h->k_init).dbs) == C) ++in_class;
-        const int launches = (in_class + kTensorsPerLaunch - 1) / kTensorsPerLaunch;
-        const int per_launch = launches ? (in_class + launches - 1) / launches : 0;
-        int64_t ws_off = 0;
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
             const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
             const int64_t ws_here = ws_off;
             if (span) ws_off += span_ws_bytes(&t, h);
-            if (chunks_for(g.dbs) != C) continue;
+            if (cls[i] != ci) continue;
             const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
             if (count == per_launch || items + nb > 0x7fffffff) {
-                const int rc = flush();
+                const int rc = close();
                 if (rc) return rc;
             }
-            TensorDesc &D = P.t[count];
+            if (count == 0) {
+                plan.emplace_back();
+                plan.back().C = classes[ci];
+            }
+            TensorDesc &D = plan.back().P.t[count];
             D.p = t.p;
             D.g = t.g;
             D.err = t.error;
@@ -778,8 +800,28 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
             ++count;
         }
-        const int rc = flush();
+        const int rc = close();
         if (rc) return rc;
+    }
+
+    for (const PlannedLaunch &L : plan) {
+        const FusedParams &P = L.P;
+        const unsigned grid = (unsigned)P.total_items;
+        const bool bf16 = h->dtype == MA_BF16;
+        int rc = 0;
+        if (dense) {
+            rc = bf16 ? launch_fused_dense_bf16(L.C, grid, P.L.total, s, P)
+                      : launch_fused_dense_f32(L.C, grid, P.L.total, s, P);
+        } else if (!span) {
+            rc = bf16 ? launch_fused_bf16(L.C, grid, P.L.total, s, P)
+                      : launch_fused_f32(L.C, grid, P.L.total, s, P);
+        } else {
+            const int passes[2] = {alpha > 0.0 ? 1 : 4, alpha > 0.0 ? 2 : 3};
+            for (int i = 0; i < 2 && rc == 0; ++i)
+                rc = bf16 ? launch_span_bf16(L.C, passes[i], grid, P.L.total, s, P)
+                          : launch_span_f32(L.C, passes[i], grid, P.L.total, s, P);
+        }
+        if (rc) return rc;  // the runtime refused a launch: earlier launches of the call stand
     }
     return 0;
 }

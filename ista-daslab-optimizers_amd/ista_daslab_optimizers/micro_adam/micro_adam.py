@@ -1,206 +1,168 @@
-"""MicroAdam on MI355X: the optimizer of ista_daslab_optimizers/micro_adam/micro_adam.py with
-the same constructor, attributes and per-parameter state, driving gfx950 HIP kernels through
-libmicroadam_hip.so.
+"""MicroAdam on MI355X.
 
-Two routes compute the same step (reference micro_adam.py:146-328):
-  * fused: one kernel pass per top-k block does Qinv + add, block top-k, window write,
-    requantisation, window -> Adam direction and the parameter update.  Taken for tensors
-    the kernel's layout conditions admit (see ma_fused_step in include/microadam_hip.h)
-    when alpha == 0.
-  * op by op: the reference's own sequence of extension calls, each a HIP kernel, with the
-    stock torch ops of the sequence (abs/topk, min/max, add_) replaced by kernels as well.
-    Taken for everything else (alpha > 0, alpha == -2, odd quantisation block sizes,
-    logging steps).
-There is no CPU or pure-PyTorch route; a missing library or a CPU tensor raises.
+Same class name, constructor, attributes and per-parameter state as the optimizer of
+ista_daslab_optimizers/micro_adam/micro_adam.py (constructor :14, state :61-94); the step itself
+is carried out by gfx950 HIP kernels of libmicroadam_hip.so.  Every tensor of a step takes one
+of four routes, all of which compute micro_adam.py:146-328:
+
+  fused            ma_fused_step            alpha == 0, quantisation blocks inside the top-k blocks
+  fused, densified ma_fused_step_densified  0 < alpha < 1, same layout
+  spanning         ma_spanning_step         0 <= alpha < 1, quantisation blocks at least as long
+                                            as the top-k blocks
+  op by op         one kernel per call of the reference's sequence: everything else
+                   (alpha == -2, other quantisation block sizes, unaligned or strided tensors)
+
+The fused routes take all their tensors in one library call per element type; what the call
+needs per tensor (seven device addresses, sizes, lr, weight decay, ring position) lives in a
+table that is built once and refreshed in place.  There is no CPU or pure-PyTorch route: a
+missing library, a missing GPU or a CPU tensor raises.
 """
 import ctypes
 import math
 import time
 
+import numpy as np
 import torch
-from torch.distributed import is_initialized, get_rank, all_reduce, ReduceOp
+import torch.distributed as dist
 
-import ista_daslab_cuda_micro_adam
-import ista_daslab_cuda_tools
+import ista_daslab_cuda_micro_adam as _ext_quant
+import ista_daslab_cuda_tools as _ext_tools
 
 from .. import _hip
-from ..tools import get_first_device, get_gpu_mem_usage, block_split, CopyDirection
+from ..tools import block_split, get_first_device, get_gpu_mem_usage
 
 try:  # logging is optional here; the reference imports wandb unconditionally (micro_adam.py:5)
     import wandb
 except Exception:  # pragma: no cover
     wandb = None
 
+OP_BY_OP, FUSED, SPANNING, FUSED_DENSIFIED = 0, 1, 2, 3
+
+# state tensors whose element type the kernels depend on (micro_adam.py:86-94)
+_TYPED_STATE = (('I', torch.int16), ('V', torch.bfloat16), ('error', torch.uint8),
+                ('min_vals', torch.bfloat16), ('max_vals', torch.bfloat16))
+
+_TENSOR_RECORD = np.dtype([(name, np.uint64 if ctype is ctypes.c_void_p else
+                            {ctypes.c_int64: np.int64, ctypes.c_double: np.float64,
+                             ctypes.c_int32: np.int32}[ctype])
+                           for name, ctype in _hip.MaTensor._fields_], align=True)
+assert _TENSOR_RECORD.itemsize == ctypes.sizeof(_hip.MaTensor)
+
+
+def _distributed():
+    return dist.is_available() and dist.is_initialized()
+
+
+class _Table:
+    """The ma_tensor records of one fused route and element type, as a ctypes array for the
+    library and a numpy view of the same memory for refreshing whole columns at once."""
+
+    def __init__(self, entries):
+        self.entries = entries
+        self.records = (_hip.MaTensor * len(entries))()
+        self.view = np.frombuffer(self.records, dtype=_TENSOR_RECORD)
+        for name in ('error', 'min_vals', 'max_vals', 'I', 'V'):
+            self.view[name] = [e.st[name].data_ptr() for e in entries]
+        self.view['d'] = [e.st['d'] for e in entries]
+        self.view['k'] = [e.st['k'] for e in entries]
+
+    def refresh(self):
+        es = self.entries
+        self.view['p'] = [e.p_addr for e in es]
+        self.view['g'] = [e.g_addr for e in es]
+        self.view['lr'] = [e.lr for e in es]
+        self.view['weight_decay'] = [e.wd for e in es]
+        self.view['index'] = [e.st['index'] for e in es]
+
+
+class _Entry:
+    """What the step knows about one parameter between steps."""
+    __slots__ = ('p', 'st', 'route', 'lr', 'wd', 'p_addr', 'g_addr')
+
+    def __init__(self, p, st, route):
+        self.p, self.st, self.route = p, st, route
+        self.lr = self.wd = 0.0
+        self.p_addr = self.g_addr = 0  # device addresses of p and p.grad in the current step
+
 
 class MicroAdam(torch.optim.Optimizer):
     def __init__(self, params, m, lr, quant_block_size, k_init=0.01, alpha=0, betas=(0.9, 0.999),
                  weight_decay=0, eps=1e-8):
-        defaults = dict(lr=lr, weight_decay=weight_decay, eps=eps, alpha=alpha)
-        super(MicroAdam, self).__init__(params, defaults)
-
+        super().__init__(params, dict(lr=lr, weight_decay=weight_decay, eps=eps, alpha=alpha))
         assert (0 <= alpha < 1) or alpha == -2, 'Alpha must be in the [0, 1) interval or -2'
 
-        self.m = m
-        self.lr = lr
+        self.m, self.lr, self.k_init, self.alpha = m, lr, k_init, alpha
         self.quant_block_size = int(quant_block_size)
-        self.k_init = k_init
-        self.alpha = alpha
-        self.weight_decay = weight_decay
-        self.beta1 = betas[0]
-        self.beta2 = betas[1]
-        self.eps = eps
+        self.weight_decay, self.eps = weight_decay, eps
+        self.beta1, self.beta2 = betas
+        self.densify_update_using_ef = alpha > 0
+        self.densify_update_using_quant_error = alpha == -2
 
-        self.densify_update_using_ef = (self.alpha > 0)
-        self.densify_update_using_quant_error = (self.alpha == -2)
-
-        self.model_size = sum([p.numel() for group in self.param_groups for p in group['params']])
-
-        self.steps = 0  # how many optimization steps were performed so far
+        every = [p for group in self.param_groups for p in group['params']]
+        self.model_size = sum(p.numel() for p in every)
+        self.steps = 0
         self.log_interval = 100
         self.device = get_first_device()
         self._is_state_initialized = False
+
+        # launch geometry the reference asks its extension for (micro_adam.py:39-44)
         self.shared_memory_carveout = 100
-        self.blocks = ista_daslab_cuda_tools.get_sm_count() * int(100 / self.shared_memory_carveout)
+        share = int(100 / self.shared_memory_carveout)
+        self.blocks = _ext_tools.get_sm_count() * share
         self.threads = 512
+        self.max_floats = _ext_tools.get_max_floats_for_shared_memory_per_thread_block()
+        self.d_block_size = self.max_floats // 2 // share
 
-        self.max_floats = ista_daslab_cuda_tools.get_max_floats_for_shared_memory_per_thread_block()
-        self.d_block_size = self.max_floats // 2 // int(100 / self.shared_memory_carveout)
+        # how many tensors of each size there are: overall, and per rank once the first step has
+        # seen which of them this rank holds (micro_adam.py:46-57, :107-114)
+        ranks = dist.get_world_size() if _distributed() else 1
+        self.fsdp_dict_size_count = [{} for _ in range(ranks)]
+        self.dict_size_count = {}
+        for p in every:
+            self.dict_size_count[p.numel()] = 1 + self.dict_size_count.get(p.numel(), 0)
 
-        if torch.distributed.is_available() and torch.distributed.is_initialized():
-            self.fsdp_dict_size_count = [{} for _ in range(torch.distributed.get_world_size())]
-        else:
-            self.fsdp_dict_size_count = [{}]
-
-        self.dict_size_count = {}  # key = layer size, value = how many layers of that size the model has
-        for param in self.param_groups:
-            for p in param['params']:
-                size = p.numel()
-                self.dict_size_count[size] = 1 + self.dict_size_count.get(size, 0)
-
-        # not in the reference: route selection and the cached descriptor table of the fused step
+        # not in the reference: route selection and the tables of the fused routes
         self.use_fused = True
-        self._fused_cache = None
-        self._route = {}
+        self._entries = {}     # parameter -> _Entry (holds the parameter, so ids are not reused)
+        self._tables = {}      # (route, dtype) -> _Table
+        self._walk = None      # per parameter group: (group, its parameter list, their entries)
         self._workspace = None  # device scratch of the spanning route, grown on demand
 
     # ------------------------------------------------------------------ state (micro_adam.py:61-94)
     def _initialize_parameter_state(self, p, lr, wd):
-        layer_size = p.numel()
+        d = p.numel()
         st = self.state[p]
-
-        rank = torch.distributed.get_rank() if (torch.distributed.is_available() and torch.distributed.is_initialized()) else 0
-
+        rank = dist.get_rank() if _distributed() else 0
         if self.densify_update_using_quant_error:
             st['quant_err'] = torch.zeros_like(p)
 
-        count = self.fsdp_dict_size_count[rank].get(layer_size, 1)
-        st['blocks'] = max(1, int(math.floor(self.blocks * layer_size * count / self.model_size)))
+        same_size = self.fsdp_dict_size_count[rank].get(d, 1)
+        st['blocks'] = max(1, int(math.floor(self.blocks * d * same_size / self.model_size)))
+        st['lr'], st['weight_decay'], st['d'] = lr, wd, d
 
-        st['lr'] = lr
-        st['weight_decay'] = wd
-        st['d'] = layer_size
+        # top-k blocks: full ones of d_block_size and a shorter last one starting at d_index_topk
+        dbs = min(d, self.d_block_size)
+        full, tail_start = block_split(d, dbs)
+        per_full = int(math.ceil(dbs * self.k_init))
+        per_tail = int(math.ceil((d - tail_start) * self.k_init))
+        st['d_block_size'] = dbs
+        st['topk_full_blocks_count'], st['d_index_topk'] = full, tail_start
+        st['k_block_size_many'], st['k_block_size_few'] = per_full, per_tail
+        st['k_index'] = full * per_full
+        st['k'] = full * per_full + per_tail
 
-        ##### variables for Top-K: d_index_topk is the index where the last, smaller topk block starts
-        st['d_block_size'] = layer_size if layer_size < self.d_block_size else self.d_block_size
-        st['topk_full_blocks_count'], st['d_index_topk'] = block_split(st['d'], st['d_block_size'])
-        st['k_block_size_many'] = int(math.ceil(st['d_block_size'] * self.k_init))
-        st['k_block_size_few'] = int(math.ceil((st['d'] - st['d_index_topk']) * self.k_init))  # 0 for d % self.d_block_size = 0
-        st['k_index'] = st['topk_full_blocks_count'] * st['k_block_size_many']
-        st['k'] = st['k_block_size_many'] * st['topk_full_blocks_count'] + st['k_block_size_few']
+        # the window: m rows of k (block-relative index, value) pairs, written round robin
+        st['index'] = 0
+        st['I'] = torch.zeros(self.m, st['k'], dtype=torch.int16, device=p.device)
+        st['V'] = torch.zeros(self.m, st['k'], dtype=torch.bfloat16, device=p.device)
 
-        ##### variables for the ring buffer
-        st['index'] = 0  # the position to place a new gradient at
-        st['I'] = torch.zeros(self.m, st['k'], dtype=torch.int16, device=p.device)  # 2mk bytes
-        st['V'] = torch.zeros(self.m, st['k'], dtype=torch.bfloat16, device=p.device)  # 2mk bytes
+        # 4-bit error feedback with one (min, max) pair per quantisation block
+        q_full, q_tail_start = block_split(d, self.quant_block_size)
+        st['quant_full_blocks_count'], st['d_index_quant'] = q_full, q_tail_start
+        st['error'] = torch.zeros(int(math.ceil(d / 2)), dtype=torch.uint8, device=p.device)
+        st['min_vals'] = torch.zeros(q_full + 1, dtype=torch.bfloat16, device=p.device)
+        st['max_vals'] = torch.zeros(q_full + 1, dtype=torch.bfloat16, device=p.device)
 
-        ### variables for error feedback: d_index_quant is the index where the last, smaller quantization block starts
-        st['quant_full_blocks_count'], st['d_index_quant'] = block_split(st['d'], self.quant_block_size)
-        st['error'] = torch.zeros(int(math.ceil(st['d'] / 2)), dtype=torch.uint8, device=p.device)  # ceil(d/2) bytes
-        st['min_vals'] = torch.zeros(st['quant_full_blocks_count'] + 1, dtype=torch.bfloat16, device=p.device)
-        st['max_vals'] = torch.zeros(st['quant_full_blocks_count'] + 1, dtype=torch.bfloat16, device=p.device)
-
-    # ------------------------------------------------------------------ step (micro_adam.py:96-144)
-    @torch.no_grad()
-    def step(self, closure=None):
-        self.steps += 1
-
-        loss = None
-        if closure is not None:
-            with torch.enable_grad():
-                loss = closure()
-
-        if self.steps == 1:
-            rank = torch.distributed.get_rank() if (torch.distributed.is_available() and torch.distributed.is_initialized()) else 0
-            for param in self.param_groups:
-                for p in param['params']:
-                    if p is not None:
-                        size = p.numel()
-                        if size > 0:
-                            self.fsdp_dict_size_count[rank][size] = 1 + self.fsdp_dict_size_count[rank].get(size, 0)
-
-        time_start = time.time()
-
-        norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe = 0, 0, 0, 0, 0, 0
-        logging_step = self._logging_active() and self.steps % self.log_interval == 0
-
-        fused, spanning, dense = [], [], []  # (p, st, lr, wd)
-        log_after = []  # tensors a fused kernel steps on a logging step: metrics taken afterwards
-        for group in self.param_groups:
-            lr = group['lr']
-            wd = group.get('weight_decay', self.weight_decay)
-
-            for p in group['params']:
-                if p.grad is None:
-                    continue
-
-                if p is None:
-                    continue
-
-                st = self.state[p]
-                if len(st) == 0:
-                    self._check_param(p)
-                    self._initialize_parameter_state(p, lr, wd)
-                self._repair_state(st)
-
-                route = self._fusable(p, st) if self.use_fused else 0
-                if logging_step and not (route in (1, 2) and self.alpha == 0):
-                    # with alpha != 0 the update holds a term that no state keeps: op by op
-                    route = 0
-                if route:
-                    if logging_step:
-                        norm_g += p.grad.view(-1).norm(p=2) ** 2  # the spanning route overwrites g
-                        log_after.append((p, st))
-                    (fused, spanning, dense)[route - 1].append((p, st, lr, wd))
-                    continue
-
-                nqe, ng, nu, ne, sp_u, sp_qe = self.update_step(p, lr, wd, logging_step)
-                norm_qe += nqe
-                norm_g += ng
-                norm_u += nu
-                norm_e += ne
-                sparsity_u += sp_u
-                sparsity_qe += sp_qe
-
-        if fused:
-            self._fused_step(fused)
-        if spanning:
-            self._fused_step(spanning, spanning=True)
-        if dense:
-            self._fused_step(dense, dense=True)
-        for p, st in log_after:
-            nu, ne, sp_u = self._metrics_after_fused_step(p, st)
-            norm_u += nu
-            norm_e += ne
-            sparsity_u += sp_u
-
-        time_end = time.time()
-        elapsed_step = time_end - time_start
-        if logging_step:
-            self._log(norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step)
-
-        return loss
-
-    # ------------------------------------------------------------------ fused route
     @staticmethod
     def _check_param(p):
         if not p.is_cuda:
@@ -208,17 +170,287 @@ class MicroAdam(torch.optim.Optimizer):
         if p.dtype not in (torch.float32, torch.bfloat16):
             raise TypeError(f"MicroAdam takes float32 or bfloat16 parameters, got {p.dtype}")
 
-    _STATE_DTYPES = (('I', torch.int16), ('V', torch.bfloat16), ('error', torch.uint8),
-                     ('min_vals', torch.bfloat16), ('max_vals', torch.bfloat16))
-
-    @classmethod
-    def _repair_state(cls, st):
-        # Frameworks that reload or re-type optimizer state cast every state tensor to the
-        # parameter's dtype (the reference repairs st['I'] for this reason,
-        # micro_adam.py:175-178); the kernels need the declared types back.
-        for key, dtype in cls._STATE_DTYPES:
+    def _repair_state(self, st):
+        """Frameworks that reload or re-type optimizer state cast every state tensor to the
+        parameter's dtype (the reference repairs st['I'] for this reason, micro_adam.py:175-178);
+        the kernels need the declared types back.  True if a tensor was replaced."""
+        replaced = False
+        for key, dtype in _TYPED_STATE:
             if st[key].dtype != dtype:
                 st[key] = st[key].to(dtype)
+                replaced = True
+        return replaced
+
+    def _entry(self, p, lr, wd):
+        """State of p (created at first touch, micro_adam.py:158-160) and its cached route."""
+        st = self.state[p]
+        if len(st) == 0:
+            self._check_param(p)
+            self._initialize_parameter_state(p, lr, wd)
+        repaired = self._repair_state(st)
+        e = self._entries.get(p)
+        if e is None or e.st is not st or repaired:
+            e = self._entries[p] = _Entry(p, st, self._static_route(p, st))
+            self._tables.clear()
+        return e
+
+    # ------------------------------------------------------------------ routes
+    def _static_route(self, p, st):
+        """The route the tensor's sizes and the hyper-parameters admit (the conditions of
+        ma_fused_step / ma_spanning_step in include/microadam_hip.h), checked by the library
+        itself where it offers the check; what depends on this step's buffers is _fusable's."""
+        if not 0 <= self.alpha < 1 or self.m > _hip.MA_MAX_WINDOW:
+            return OP_BY_OP
+        # state made for another top-k block size (a checkpoint from other hardware) runs op by
+        # op from its stored geometry; the fused kernels derive theirs from self.d_block_size
+        d, dbs = st['d'], st['d_block_size']
+        expect_k = (int(math.ceil(dbs * self.k_init)) * (d // dbs)
+                    + int(math.ceil((d - d // dbs * dbs) * self.k_init)))
+        if dbs != min(d, self.d_block_size) or st['k'] != expect_k:
+            return OP_BY_OP
+        probe = _hip.MaTensor()
+        for name in ('p', 'g'):
+            setattr(probe, name, 256)  # stands for any 16-byte aligned address
+        for name, _ in _TYPED_STATE:
+            setattr(probe, name, st[name].data_ptr())
+        probe.d, probe.k, probe.index = d, st['k'], 0
+        h = self._hyper(p.dtype, max(self.steps, 1))
+        if _hip.lib.ma_fused_step_check(ctypes.byref(probe), ctypes.byref(h)) == 0:
+            return FUSED if self.alpha == 0 else FUSED_DENSIFIED
+        if _hip.lib.ma_spanning_step_check(ctypes.byref(probe), ctypes.byref(h),
+                                           float(self.alpha)) == 0:
+            return SPANNING
+        return OP_BY_OP
+
+    def _fusable(self, p, st):
+        """Route p takes in a step with its current gradient: 0 op by op, 1 fused, 2 spanning,
+        3 fused densified."""
+        g = p.grad
+        if g.dtype != p.dtype or not p.is_contiguous() or not g.is_contiguous():
+            return OP_BY_OP
+        if (p.data_ptr() | g.data_ptr()) & 15:
+            return OP_BY_OP
+        e = self._entries.get(p)
+        if e is None or e.st is not st:
+            return self._static_route(p, st)
+        return e.route
+
+    def _hyper(self, dtype, t):
+        return _hip.MaHyper(t, self.m, _hip.MA_BF16 if dtype == torch.bfloat16 else _hip.MA_F32,
+                            self.quant_block_size, self.d_block_size, self.k_init, self.beta1,
+                            self.beta2, self.eps)
+
+    # ------------------------------------------------------------------ step (micro_adam.py:96-144)
+    @torch.no_grad()
+    def step(self, closure=None):
+        self.steps += 1
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+
+        if self.steps == 1:
+            mine = self.fsdp_dict_size_count[dist.get_rank() if _distributed() else 0]
+            for group in self.param_groups:
+                for p in group['params']:
+                    if p is not None and p.numel() > 0:
+                        mine[p.numel()] = 1 + mine.get(p.numel(), 0)
+
+        started = time.time()
+        logging_step = self._logging_active() and self.steps % self.log_interval == 0
+        totals = dict(norm_qe=0, norm_g=0, norm_u=0, norm_e=0, sparsity_u=0, sparsity_qe=0)
+        batches = {}  # (route, dtype) -> entries, in parameter order
+        fused_allowed = self.use_fused and not (logging_step and self.alpha != 0)
+        for group, plist, entries in self._groups():
+            lr = group['lr']
+            wd = group.get('weight_decay', self.weight_decay)
+            for i, p in enumerate(plist):
+                g = None if p is None else p.grad
+                if g is None:
+                    continue
+                e = entries[i]
+                if e is None or e.st['I'].dtype is not torch.int16:
+                    e = entries[i] = self._entry(p, lr, wd)
+                # what this step's buffers admit: same element type, dense, 16-byte aligned
+                # (with alpha != 0 a logging step goes op by op: the update then holds a term
+                # that no state keeps)
+                route = OP_BY_OP
+                if (fused_allowed and e.route and g.dtype is p.dtype and g.is_contiguous()
+                        and p.is_contiguous()):
+                    e.p_addr, e.g_addr = p.data_ptr(), g.data_ptr()
+                    if not (e.p_addr | e.g_addr) & 15:
+                        route = e.route
+                if route == OP_BY_OP:
+                    for key, value in self.update_step(p, lr, wd, logging_step).items():
+                        totals[key] += value
+                    continue
+                e.lr, e.wd = lr, wd
+                if logging_step:  # before the step: the spanning route overwrites g
+                    totals['norm_g'] += g.view(-1).norm(p=2) ** 2
+                batch = batches.get((route, p.dtype))
+                if batch is None:
+                    batch = batches[(route, p.dtype)] = []
+                batch.append(e)
+
+        for (route, dtype), entries in batches.items():
+            self._fused_step(route, dtype, entries)
+            if logging_step:
+                for e in entries:
+                    for key, value in self._metrics_after_fused_step(e.p, e.st).items():
+                        totals[key] += value
+
+        if logging_step:
+            self._log(totals['norm_qe'], totals['norm_g'], totals['norm_u'], totals['norm_e'],
+                      totals['sparsity_u'], totals['sparsity_qe'], time.time() - started)
+        return loss
+
+    def _groups(self):
+        """The parameter groups with the cached entries of their parameters, rebuilt when a
+        group was added or a group's parameter list replaced or resized."""
+        walk = self._walk
+        groups = self.param_groups
+        if walk is None or len(walk) != len(groups) or any(
+                w[0] is not g or w[1] is not g['params'] or len(w[2]) != len(w[1])
+                for w, g in zip(walk, groups)):
+            walk = self._walk = [(g, g['params'], [self._entries.get(p) for p in g['params']])
+                                 for g in groups]
+        return walk
+
+    # ------------------------------------------------------------------ fused routes
+    def _fused_step(self, route, dtype, entries):
+        table = self._tables.get((route, dtype))
+        if table is None or len(table.entries) != len(entries) or any(
+                a is not b for a, b in zip(table.entries, entries)):
+            table = self._tables[(route, dtype)] = _Table(list(entries))
+        table.refresh()
+        n, h, stream = len(entries), self._hyper(dtype, self.steps), _hip.stream_ptr()
+        if route == FUSED:
+            rc = _hip.lib.ma_fused_step(table.records, n, ctypes.byref(h), stream)
+            _hip.check(rc, "ma_fused_step")
+        elif route == FUSED_DENSIFIED:
+            rc = _hip.lib.ma_fused_step_densified(table.records, n, ctypes.byref(h),
+                                                  float(self.alpha), stream)
+            _hip.check(rc, "ma_fused_step_densified")
+        else:
+            need = _hip.lib.ma_spanning_step_workspace(table.records, n, ctypes.byref(h))
+            device = entries[0].p.device
+            ws = self._workspace
+            if ws is None or ws.numel() < need or ws.device != device:
+                ws = self._workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+            rc = _hip.lib.ma_spanning_step(table.records, n, ctypes.byref(h), float(self.alpha),
+                                           ws.data_ptr(), ws.numel(), stream)
+            _hip.check(rc, "ma_spanning_step")
+        for e in entries:  # micro_adam.py:211
+            e.st['index'] = (e.st['index'] + 1) % self.m
+
+    # ------------------------------------------------------------------ op-by-op route (micro_adam.py:146-328)
+    @torch.no_grad()
+    def update_step(self, p, lr, wd, logging_step=False):
+        """One tensor through the reference's own sequence of device operations.  Returns the
+        logging sums of this tensor (all zero unless logging_step)."""
+        out = dict(norm_qe=0, norm_g=0, norm_u=0, norm_e=0, sparsity_u=0, sparsity_qe=0)
+        st = self._entry(p, lr, wd).st
+        acc = p.grad.view(-1)  # the gradient buffer is accumulator, update and scratch in turn
+        d, q = st['d'], self.quant_block_size
+        error, lo, hi = st['error'], st['min_vals'], st['max_vals']
+        stream, tag = _hip.stream_ptr(), _hip.dtype_tag(acc)
+        acc_ptr = _hip.dev_ptr(acc, None, "grad")
+
+        def add_dequantised(scale):  # acc += scale * Qinv(error)
+            _ext_quant.asymm_block_quant_inv(d, q, error, lo, hi, acc, scale)
+
+        def requantise():  # statistics of acc per quantisation block, then error = Q(acc)
+            _hip.check(_hip.lib.ma_block_minmax(d, q, acc_ptr, _hip.dev_ptr(lo, torch.bfloat16, "min_vals"),
+                                                _hip.dev_ptr(hi, torch.bfloat16, "max_vals"), tag,
+                                                stream), "ma_block_minmax")
+            _ext_quant.asymm_block_quant(d, q, error, lo, hi, acc)
+
+        if logging_step:
+            out['norm_g'] = acc.norm(p=2) ** 2
+
+        # accumulator = gradient + error feedback; its block-wise top-k moves into window row
+        # `index` (selection, value gather and zeroing are one launch); the rest is requantised
+        add_dequantised(1.0)
+        row = st['index']
+        _hip.check(_hip.lib.ma_block_topk(d, st['d_block_size'], st['k_block_size_many'],
+                                          st['k_block_size_few'], acc_ptr,
+                                          _hip.dev_ptr(st['I'][row], torch.int16, "I row"),
+                                          _hip.dev_ptr(st['V'][row], torch.bfloat16, "V row"),
+                                          1, tag, stream), "ma_block_topk")
+        st['index'] = (row + 1) % self.m
+        requantise()
+
+        # decoupled weight decay goes into the update kernel unless something reads p first
+        plain = p.dtype == acc.dtype and p.is_contiguous()
+        decay_in_kernel = plain and not self.densify_update_using_quant_error
+        if wd > 0 and not decay_in_kernel:
+            p.mul_(1 - lr * wd)
+
+        if self.densify_update_using_quant_error:
+            # alpha == -2 (micro_adam.py:238-273): what quantisation lost of the accumulator goes
+            # straight into the parameters: p -= a, p += Qinv(Q(a)); quant_err keeps a - Qinv(Q(a))
+            lost = st['quant_err']
+            lost.copy_(p.grad)
+            p.sub_(p.grad)
+            acc.zero_()
+            add_dequantised(1)
+            p.add_(p.grad)
+            lost.sub_(p.grad)
+            if logging_step:
+                out['norm_qe'] = lost.norm(p=2) ** 2
+                out['sparsity_qe'] = (lost == 0).sum()
+
+        # Adam direction rebuilt from the window, plus alpha * error feedback if asked for
+        acc.zero_()
+        _ext_quant.compute_microadam_update(st['blocks'], self.threads, self.shared_memory_carveout,
+                                            self.steps, self.beta1, self.beta2, self.eps,
+                                            st['d_block_size'], st['k_block_size_many'], d, self.m,
+                                            st['k'], st['I'], st['V'], acc)
+        if self.densify_update_using_ef:
+            add_dequantised(self.alpha)
+
+        if plain:
+            decay = wd > 0 and decay_in_kernel
+            _hip.check(_hip.lib.ma_param_update(d, _hip.dev_ptr(p, None, "p"), acc_ptr, -lr,
+                                                1 if decay else 0, 1 - lr * wd, tag, stream),
+                       "ma_param_update")
+        else:
+            p.add_(p.grad, alpha=-lr)
+
+        if logging_step:
+            out['norm_u'] = acc.norm(p=2) ** 2
+            out['sparsity_u'] = (acc == 0).sum()
+
+        if self.densify_update_using_ef:
+            # the share of the error feedback that went into the update leaves it
+            acc.zero_()
+            add_dequantised(1 - self.alpha)
+            requantise()
+
+        if logging_step:
+            acc.zero_()
+            add_dequantised(1.0)
+            out['norm_e'] = acc.norm(p=2) ** 2
+        return out
+
+    def _metrics_after_fused_step(self, p, st):
+        """norm_u, norm_e and the update's zero count (micro_adam.py:306-308, :320-324) for a
+        tensor that a fused kernel has just stepped with alpha == 0: the update is rebuilt from
+        the window (which already holds this step's row, as at micro_adam.py:277-291) and the
+        error norm from the stored error feedback, both in p.grad, which the step leaves as
+        scratch like the reference does (:276, :321)."""
+        scratch = p.grad.view(-1)
+        scratch.zero_()
+        _ext_quant.compute_microadam_update(st['blocks'], self.threads, self.shared_memory_carveout,
+                                            self.steps, self.beta1, self.beta2, self.eps,
+                                            st['d_block_size'], st['k_block_size_many'], st['d'],
+                                            self.m, st['k'], st['I'], st['V'], scratch)
+        out = dict(norm_u=scratch.norm(p=2) ** 2, sparsity_u=(scratch == 0).sum())
+        scratch.zero_()
+        _ext_quant.asymm_block_quant_inv(st['d'], self.quant_block_size, st['error'], st['min_vals'],
+                                         st['max_vals'], scratch, 1.0)
+        out['norm_e'] = scratch.norm(p=2) ** 2
+        return out
 
     # ------------------------------------------------------------------ checkpointing
     def state_dict(self):
@@ -243,252 +475,12 @@ class MicroAdam(torch.optim.Optimizer):
             if saved is None:
                 continue
             st = self.state[p]
-            for key, dtype in self._STATE_DTYPES:
+            for key, dtype in _TYPED_STATE:
                 if key in saved and torch.is_tensor(saved[key]) and saved[key].dtype == dtype:
                     st[key] = saved[key].to(device=p.device, copy=True)
-        self._fused_cache = None
-
-    def _fusable(self, p, st):
-        """0: op-by-op route; 1: ma_fused_step (alpha == 0, quantisation blocks inside the top-k
-        blocks); 2: ma_spanning_step (0 <= alpha < 1, quantisation blocks at least as long as the
-        top-k blocks); 3: ma_fused_step_densified (as 1 with 0 < alpha < 1).  The conditions are
-        those of include/microadam_hip.h."""
-        if not 0 <= self.alpha < 1:
-            return 0
-        g = p.grad
-        if g.dtype != p.dtype or not p.is_contiguous() or not g.is_contiguous():
-            return 0
-        if (p.data_ptr() | g.data_ptr()) & 15:
-            return 0
-        route = self._route.get(id(p))
-        if route is None:
-            q, d, dbs = self.quant_block_size, st['d'], st['d_block_size']
-            common = (self.m <= _hip.MA_MAX_WINDOW and dbs <= 32768
-                      and (d <= self.d_block_size or dbs % 8 == 0))
-            route = 0
-            if (common and 8 <= q <= 512 and (q & (q - 1)) == 0 and d >= q
-                    and (d <= self.d_block_size or dbs % q == 0)):
-                route = 1 if self.alpha == 0 else 3
-            elif (common and q % 8 == 0 and dbs <= q < (1 << 30)
-                  and (q + dbs - 1) // dbs + 1 <= 64):
-                route = 2
-            self._route[id(p)] = route
-        return route
-
-    def _fused_step(self, items, spanning=False, dense=False):
-        n = len(items)
-        kind = 1 if spanning else 2 if dense else 0
-        key = (kind,) + tuple(id(p) for p, _, _, _ in items)
-        cache = self._fused_cache.get(kind) if self._fused_cache else None
-        if cache is None or cache[0] != key:
-            arr = (_hip.MaTensor * n)()
-            for t, (p, st, _, _) in zip(arr, items):
-                t.d = st['d']
-                t.k = st['k']
-            cache = (key, arr)
-            if self._fused_cache is None:
-                self._fused_cache = {}
-            self._fused_cache[kind] = cache
-        arr = cache[1]
-        for t, (p, st, lr, wd) in zip(arr, items):
-            t.p = p.data_ptr()
-            t.g = p.grad.data_ptr()
-            t.error = st['error'].data_ptr()
-            t.min_vals = st['min_vals'].data_ptr()
-            t.max_vals = st['max_vals'].data_ptr()
-            t.I = st['I'].data_ptr()
-            t.V = st['V'].data_ptr()
-            t.lr = lr
-            t.weight_decay = wd
-            t.index = st['index']
-        by_dtype = {}
-        for i, (p, _, _, _) in enumerate(items):
-            by_dtype.setdefault(p.dtype, []).append(i)
-        for dtype, idxs in by_dtype.items():
-            if len(idxs) == n:
-                sub, cnt = arr, n
-            else:
-                sub = (_hip.MaTensor * len(idxs))(*[arr[i] for i in idxs])
-                cnt = len(idxs)
-            h = _hip.MaHyper(self.steps, self.m, _hip.MA_BF16 if dtype == torch.bfloat16 else _hip.MA_F32,
-                             self.quant_block_size, self.d_block_size, self.k_init, self.beta1,
-                             self.beta2, self.eps)
-            if dense:
-                rc = _hip.lib.ma_fused_step_densified(sub, cnt, ctypes.byref(h), float(self.alpha),
-                                                      _hip.stream_ptr())
-                _hip.check(rc, "ma_fused_step_densified")
-                continue
-            if not spanning:
-                rc = _hip.lib.ma_fused_step(sub, cnt, ctypes.byref(h), _hip.stream_ptr())
-                _hip.check(rc, "ma_fused_step")
-                continue
-            need = _hip.lib.ma_spanning_step_workspace(sub, cnt, ctypes.byref(h))
-            ws = self._workspace
-            if ws is None or ws.numel() < need or ws.device != items[idxs[0]][0].device:
-                ws = self._workspace = torch.empty(max(need, 16), dtype=torch.uint8,
-                                                   device=items[idxs[0]][0].device)
-            rc = _hip.lib.ma_spanning_step(sub, cnt, ctypes.byref(h), float(self.alpha),
-                                            ws.data_ptr(), ws.numel(), _hip.stream_ptr())
-            _hip.check(rc, "ma_spanning_step")
-        for _, st, _, _ in items:
-            st['index'] = (st['index'] + 1) % self.m
-
-    # ------------------------------------------------------------------ op-by-op route (micro_adam.py:146-328)
-    @torch.no_grad()
-    def update_step(self, p, lr, wd, logging_step=False):
-        norm_qe, norm_g, norm_u, norm_e, sp_u, sp_qe = 0, 0, 0, 0, 0, 0
-
-        grad = p.grad.view(-1)
-
-        if logging_step:
-            norm_g = grad.norm(p=2) ** 2
-
-        st = self.state[p]
-        if len(st) == 0:
-            self._check_param(p)
-            self._initialize_parameter_state(p, lr, wd)
-
-        blocks = st['blocks']
-        d = st['d']
-        d_block_size = st['d_block_size']
-        k_block_size_many = st['k_block_size_many']
-        k_block_size_few = st['k_block_size_few']
-        k = st['k']
-
-        self._repair_state(st)
-
-        index = st['index']
-        I = st['I']
-        V = st['V']
-
-        error = st['error']
-        min_vals = st['min_vals']
-        max_vals = st['max_vals']
-        stream = _hip.stream_ptr()
-        tag = _hip.dtype_tag(grad)
-        gptr = _hip.dev_ptr(grad, None, "grad")
-
-        ##### STEP 4
-        ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, error, min_vals, max_vals, grad, 1.0)
-
-        ##### STEP 5 + 9 + 6: block top-k, V = a[I], a[I] = 0 in one launch
-        _hip.check(_hip.lib.ma_block_topk(d, d_block_size, k_block_size_many, k_block_size_few, gptr,
-                                          _hip.dev_ptr(I[index, :], torch.int16, "I row"),
-                                          _hip.dev_ptr(V[index, :], torch.bfloat16, "V row"),
-                                          1, tag, stream), "ma_block_topk")
-
-        st['index'] = (index + 1) % self.m
-
-        ##### STEP 7
-        def _update_quantization_statistics():
-            _hip.check(_hip.lib.ma_block_minmax(d, self.quant_block_size, gptr,
-                                                _hip.dev_ptr(min_vals, torch.bfloat16, "min_vals"),
-                                                _hip.dev_ptr(max_vals, torch.bfloat16, "max_vals"),
-                                                tag, stream), "ma_block_minmax")
-
-        _update_quantization_statistics()
-
-        ##### STEP 8
-        ista_daslab_cuda_micro_adam.asymm_block_quant(d, self.quant_block_size, error, min_vals, max_vals, grad)  # error = Q(a, min, max)
-
-        # weight decay step: folded into the update kernel below unless something reads p first
-        same_layout = p.dtype == grad.dtype and p.is_contiguous()
-        fold_decay = same_layout and not self.densify_update_using_quant_error
-        if wd > 0 and not fold_decay:
-            p.mul_(1 - lr * wd)
-
-        ##### NEW: densify using quant error (micro_adam.py:238-273)
-        if self.densify_update_using_quant_error:
-            quant_err = st['quant_err']
-            quant_err.zero_()
-            quant_err.add_(p.grad)
-
-            ##### STEP A
-            p.add_(p.grad, alpha=-1)
-
-            ##### STEP B
-            p.grad.zero_()  # zerorize to prepare the accumulator for Qinv
-            ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, error, min_vals, max_vals, grad, 1)
-            p.add_(p.grad)
-
-            quant_err.sub_(p.grad)
-
-            if logging_step:
-                norm_qe = quant_err.norm(p=2) ** 2
-                sp_qe = (quant_err == 0).sum()
-
-        ##### STEPS 10-11
-        grad.zero_()
-        ista_daslab_cuda_micro_adam.compute_microadam_update(blocks,  # blocks
-                                                             self.threads,  # threads
-                                                             self.shared_memory_carveout,  # carveout
-                                                             self.steps,  # optimization step
-                                                             self.beta1,  # beta1
-                                                             self.beta2,  # beta2
-                                                             self.eps,  # eps
-                                                             d_block_size,  # d_block_size
-                                                             k_block_size_many,  # k_block_size
-                                                             d,  # d
-                                                             self.m,  # m
-                                                             k,  # k
-                                                             I,  # indices
-                                                             V,  # values
-                                                             grad)  # update will be stored here
-
-        ##### if PRETRAINING #1
-        if self.densify_update_using_ef:  # we add alpha * EF to update that is stored in grad buffer
-            ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, error, min_vals, max_vals, grad, self.alpha)
-
-        # update model using MicroAdam update stored in p.grad
-        if same_layout:
-            apply_decay = wd > 0 and fold_decay
-            _hip.check(_hip.lib.ma_param_update(d, _hip.dev_ptr(p, None, "p"), gptr, -lr,
-                                                1 if apply_decay else 0, 1 - lr * wd, tag, stream),
-                       "ma_param_update")
-        else:
-            p.add_(p.grad, alpha=-lr)
-
-        if logging_step:
-            norm_u = grad.norm(p=2) ** 2
-            sp_u = (grad == 0).sum()  # check sparsity before zerorizing
-
-        ##### if PRETRAINING #2
-        if self.densify_update_using_ef:
-            grad.zero_()
-            ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, error, min_vals, max_vals, grad, 1 - self.alpha)
-
-            _update_quantization_statistics()  # step 7 again
-            ista_daslab_cuda_micro_adam.asymm_block_quant(d, self.quant_block_size, error, min_vals, max_vals, grad)  # step 8 again
-
-        # compute error norm
-        if logging_step:
-            grad.zero_()
-            ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, error, min_vals, max_vals, grad, 1.0)
-
-            norm_e = grad.norm(p=2) ** 2
-
-        return norm_qe, norm_g, norm_u, norm_e, sp_u, sp_qe
-
-    def _metrics_after_fused_step(self, p, st):
-        """norm_u, norm_e and the update's zero count (micro_adam.py:306-308, :320-324) for a
-        tensor that a fused kernel has just stepped with alpha == 0: the update is rebuilt from
-        the window (which already holds this step's row, as at micro_adam.py:277-291) and the
-        error norm from the stored error feedback, both in p.grad, which the step leaves as
-        scratch like the reference does (:276, :321)."""
-        grad = p.grad.view(-1)
-        d = st['d']
-        grad.zero_()
-        ista_daslab_cuda_micro_adam.compute_microadam_update(
-            st['blocks'], self.threads, self.shared_memory_carveout, self.steps, self.beta1,
-            self.beta2, self.eps, st['d_block_size'], st['k_block_size_many'], d, self.m, st['k'],
-            st['I'], st['V'], grad)
-        norm_u = grad.norm(p=2) ** 2
-        sp_u = (grad == 0).sum()
-        grad.zero_()
-        ista_daslab_cuda_micro_adam.asymm_block_quant_inv(d, self.quant_block_size, st['error'],
-                                                          st['min_vals'], st['max_vals'], grad, 1.0)
-        norm_e = grad.norm(p=2) ** 2
-        return norm_u, norm_e, sp_u
+        self._entries.clear()
+        self._tables.clear()
+        self._walk = None
 
     # ------------------------------------------------------------------ logging (micro_adam.py:330-350)
     @staticmethod
@@ -496,23 +488,23 @@ class MicroAdam(torch.optim.Optimizer):
         return wandb is not None and getattr(wandb, 'run', None) is not None
 
     def _log(self, norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step):
-        if self.steps % self.log_interval == 0:
-            if is_initialized():
-                sync_data = torch.tensor([norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step], dtype=torch.float,
-                                         requires_grad=False).cuda()
-                all_reduce(sync_data, op=ReduceOp.SUM)
-                norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step = sync_data
-
-            if not is_initialized() or get_rank() == 0:
-                wandb_data = {
-                    'step/optimizer_steps': self.steps,
-                    'step/gpu_mem_usage': get_gpu_mem_usage(),
-                    'step/norm_quant_err': math.sqrt(norm_qe),
-                    'step/sparsity_quant_err': sparsity_qe / self.model_size * 100.,
-                    'step/norm_g': math.sqrt(norm_g),
-                    'step/norm_u': math.sqrt(norm_u),
-                    'step/norm_error': math.sqrt(norm_e),
-                    'step/sparsity_u': sparsity_u / self.model_size * 100.,
-                    'step/elapsed_step': elapsed_step,
-                }
-                wandb.log(wandb_data, commit=False)
+        if self.steps % self.log_interval != 0:
+            return
+        sums = [norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step]
+        if _distributed():
+            buf = torch.tensor([float(x) for x in sums], dtype=torch.float).cuda()
+            dist.all_reduce(buf, op=dist.ReduceOp.SUM)
+            sums = buf.tolist()
+            if dist.get_rank() != 0:
+                return
+        norm_qe, norm_g, norm_u, norm_e, sparsity_u, sparsity_qe, elapsed_step = sums
+        percent = 100. / self.model_size
+        wandb.log({'step/optimizer_steps': self.steps,
+                   'step/gpu_mem_usage': get_gpu_mem_usage(),
+                   'step/norm_quant_err': math.sqrt(norm_qe),
+                   'step/sparsity_quant_err': sparsity_qe * percent,
+                   'step/norm_g': math.sqrt(norm_g),
+                   'step/norm_u': math.sqrt(norm_u),
+                   'step/norm_error': math.sqrt(norm_e),
+                   'step/sparsity_u': sparsity_u * percent,
+                   'step/elapsed_step': elapsed_step}, commit=False)
