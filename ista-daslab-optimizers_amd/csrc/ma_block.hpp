@@ -266,14 +266,13 @@ struct FusedBlock {
     }
 
     // ---- the whole window of the block into registers, for the general window stage
-    // Entries travel two per 32-bit load, so every row of the block has to start on a 4-byte
-    // boundary and hold an even number of entries; otherwise, or when the window has more
-    // than kHold steps, the stage streams the entries as window_accumulate does.
+    // Entries travel two per 32-bit load (from any 2-byte boundary), so a row of the block has
+    // to hold an even number of entries; otherwise, or when the window has more than kHold
+    // steps, the stage streams the entries as window_accumulate does.
     __device__ __forceinline__ bool can_hold(const BlockGeo &G) const {
         const int pairs = G.kb >> 1;
         const int trips = (pairs + kWG - 1) / kWG;
-        return HOLD && P.L.cell_bytes == 0 && ((G.kb | G.D.k | G.col0) & 1) == 0 &&
-               (((uintptr_t)G.D.I | (uintptr_t)G.D.V) & 3) == 0 && P.W.rows * trips <= kHold;
+        return HOLD && P.L.cell_bytes == 0 && (G.kb & 1) == 0 && P.W.rows * trips <= kHold;
     }
 
     // current == false: the older rows, from memory (can be asked for before the selection);
@@ -283,9 +282,12 @@ struct FusedBlock {
         if (!holding) return;
         const int pairs = G.kb >> 1;
         const int trips = (pairs + kWG - 1) / kWG;
-        const uint32_t *I2 = reinterpret_cast<const uint32_t *>(G.D.I + G.col0);
-        const uint32_t *V2 = reinterpret_cast<const uint32_t *>(G.D.V + G.col0);
-        const int64_t k2 = G.D.k >> 1;
+        // (a pair may start on any 2-byte boundary: the hardware takes unaligned loads)
+        struct __attribute__((packed, aligned(2))) Pair {
+            uint32_t w;
+        };
+        const int16_t *Ib = G.D.I + G.col0;
+        const uint16_t *Vb = G.D.V + G.col0;
         int row = 0, it = 0;  // uniform
 #pragma unroll
         for (int s = 0; s < kHold; ++s) {
@@ -301,8 +303,9 @@ struct FusedBlock {
                         hI[s] = reinterpret_cast<const uint32_t *>(sel_idx)[w];
                         hV[s] = reinterpret_cast<const uint32_t *>(sel_val)[w];
                     } else if (!current && !from_lds) {
-                        hI[s] = I2[row * k2 + w];
-                        hV[s] = V2[row * k2 + w];
+                        const int64_t at = (int64_t)row * G.D.k + 2 * w;
+                        hI[s] = reinterpret_cast<const Pair *>(Ib + at)->w;
+                        hV[s] = reinterpret_cast<const Pair *>(Vb + at)->w;
                     }
                 }
                 if (++it == trips) {
