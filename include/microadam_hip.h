@@ -216,6 +216,42 @@ int ma_spanning_step_check(const ma_tensor *tensor /* host */, const ma_hyper *h
 int ma_spanning_step_static(const ma_tensor *tensors /* host */, int n_tensors,
                              const ma_hyper *hyper /* host */, double alpha, void *stream);
 
+/* ma_fused_step for alpha == -2 (densify_update_using_quant_error, MA:238-273), same conditions,
+ * still one pass per top-k block: with the residual a and the new error feedback e in
+ * registers, p = p * (1 - lr * wd) (MA:234-235), p = p - a (MA:264), p = p + Qinv(e) (MA:269),
+ * each rounded to the parameter's type, then the Adam step as for alpha == 0.  st['quant_err']
+ * (MA:258-270, read by the logged norms only) is not written. */
+int ma_fused_step_quant_err(const ma_tensor *tensors /* host */, int n_tensors,
+                            const ma_hyper *hyper /* host */, void *stream);
+
+/* ---- logging steps (MA:155-156, :271-272, :306-308, :320-324, summed in _log's order MA:328) */
+#define MA_ROUTE_FUSED 0     /* as ma_fused_step */
+#define MA_ROUTE_DENSIFIED 1 /* as ma_fused_step_densified */
+#define MA_ROUTE_SPANNING 2  /* as ma_spanning_step */
+#define MA_ROUTE_QUANT_ERR 3 /* as ma_fused_step_quant_err */
+
+/* One step as the entry point named by `route` takes it (same arguments, conditions and
+ * results; alpha, workspace and workspace_bytes as that entry point has them, else ignored),
+ * that also forms the sums the reference logs every log_interval steps, as side reductions of
+ * the same kernels: every top-k block leaves 8 floats in `partials`, a last kernel adds them
+ * in double, in a fixed order, and ADDS the totals to sums[0..5] (sums[6..7] unused):
+ *   sums[0] |quant_err|^2 (MA:271; route QUANT_ERR only, else 0)   sums[1] |g|^2 (MA:155-156)
+ *   sums[2] |u|^2 (MA:307)      sums[3] |Qinv(error)|^2 after the step (MA:320-324)
+ *   sums[4] zeros of u (MA:308) sums[5] zeros of quant_err (MA:272)
+ * taken from the values as the reference's buffers hold them (rounded to the gradient's
+ * type).  Equal inputs give equal bits.
+ * partials: device, at least ma_logged_step_partials() floats, contents need not survive the
+ * call.  sums: device, 8 doubles, cleared by the caller before the first call of the step. */
+int ma_logged_step(int route, const ma_tensor *tensors /* host */, int n_tensors,
+                   const ma_hyper *hyper /* host */, double alpha, void *workspace,
+                   int64_t workspace_bytes, float *partials, int64_t n_partials, double *sums,
+                   void *stream);
+
+/* Floats of `partials` ma_logged_step needs for this list (8 per top-k block); -1 on bad
+ * arguments.  Host-only. */
+int64_t ma_logged_step_partials(const ma_tensor *tensors /* host */, int n_tensors,
+                                const ma_hyper *hyper /* host */);
+
 /* ---- ista_daslab_cuda_sparse_mfac: the kernels that share the window layout -------------- */
 /* Sparse M-FAC (sparse_mfac/sparse_core_mfac_w_ef.py, SC below) keeps its m gradients in the
  * same I (int16, block-relative) / V layout as MicroAdam's window; its values are bf16 or, with

@@ -77,7 +77,25 @@ struct FusedParams {
     int32_t q_span;   // quantisation block length, a multiple of 8
     float alpha;      // share of the dequantised error feedback added to the update
     float keep;       // (float)(1 - alpha): share that stays in the error feedback
+    // logging steps (kernels compiled with kAuxLog): kMetricSlots floats per work item
+    float *metrics;
 };
+
+// Extras of a block kernel (template parameter AUX, a set of bits).  Kernels with extras run
+// rarely or on request, and are compiled for any quantisation group with the register budget
+// of two workgroups per CU.
+//   kAuxLog: a logging step (MA:155-156, :271-272, :306-308, :320-324): every block leaves the
+//            sums of its elements in its metrics slot, in the order of the reference's return
+//            value (MA:328): |quant_err|^2, |g|^2, |u|^2, |Qinv(e)|^2, zeros of u, zeros of
+//            quant_err (the counts as floats; two unused floats pad the slot to 32 bytes).
+//            The values are summed as the reference's buffers hold them (rounded to the
+//            gradient's type), in fp32 and in a fixed order.
+//   kAuxQuantErr: alpha == -2 (MA:238-273): what the quantisation of the residual loses goes
+//            straight into the parameters, p = p - a, then p = p + Qinv(e) (each rounded to
+//            the parameter's type) before the Adam step.
+constexpr int kAuxLog = 1, kAuxQuantErr = 2;
+constexpr int kMetricSlots = 8;
+enum { kMtQuantErr = 0, kMtGrad = 1, kMtUpdate = 2, kMtError = 3, kMtUpdateZeros = 4, kMtQuantErrZeros = 5 };
 
 template <class R>
 struct RawChunk;
@@ -106,6 +124,10 @@ struct RawChunk<RegsBF16<C>> {
             v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
         }
     }
+    __device__ __forceinline__ void from_float(const float (&v)[8]) {
+        q = make_uint4(f2bf_pair(v[0], v[1]), f2bf_pair(v[2], v[3]), f2bf_pair(v[4], v[5]),
+                       f2bf_pair(v[6], v[7]));
+    }
 };
 template <int C>
 struct RawChunk<RegsF32<C>> {
@@ -123,6 +145,10 @@ struct RawChunk<RegsF32<C>> {
     __device__ __forceinline__ void to_float(float (&v)[8]) const {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = v_[i];
+    }
+    __device__ __forceinline__ void from_float(const float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v_[i] = v[i];
     }
 };
 
@@ -160,10 +186,72 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
 //   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
 //   HOLD: the general window stage may keep the block's window entries in registers (40 of
 //         them), for kernels compiled with the register budget of two workgroups per CU.
-template <class R, bool FULL, int QL, bool HOLD = false>
+template <class R, bool FULL, int QL, bool HOLD = false, int AUX = 0>
 struct FusedBlock {
     typedef typename R::elem_t elem_t;
     static constexpr int C = R::kC;
+    static constexpr bool LOG = (AUX & kAuxLog) != 0, QE = (AUX & kAuxQuantErr) != 0;
+
+    // ---- the sums of a logging step: per thread, then per workgroup in log_flush
+    float mt[LOG ? 6 : 1];
+
+    __device__ __forceinline__ void log_square(int which, float v) {
+        if constexpr (LOG) {
+            const float sq = v * v;
+            mt[which] = mt[which] + sq;
+        }
+    }
+    __device__ __forceinline__ void log_zero(int which, float v) {
+        if constexpr (LOG) mt[which] = mt[which] + (v == 0.0f ? 1.0f : 0.0f);
+    }
+    // the update of 8 coordinates of which the first `valid` belong to the block
+    __device__ __forceinline__ void log_update(const float (&uv)[8], int valid) {
+        if constexpr (LOG) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                if (e < valid) {
+                    log_square(kMtUpdate, uv[e]);
+                    log_zero(kMtUpdateZeros, uv[e]);
+                }
+            }
+        }
+    }
+
+    // the error feedback just formed: codes (as floats) of 8 elements against (mn, u)
+    __device__ __forceinline__ void log_error(const float (&cf)[8], float mnf, float u, int valid) {
+        if constexpr (LOG) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) {
+                float deq = cf[e] * u;
+                deq = deq + mnf;
+                if (e < valid) log_square(kMtError, to_elem(0.0f + deq));
+            }
+        }
+    }
+
+    // The workgroup's sums of the components in `mask` go to the block's slot (the other
+    // components belong to another pass over the same blocks): lanes, then waves, in a fixed
+    // order.  Every thread calls it, at the end of the kernel.
+    __device__ __forceinline__ void log_flush(int item, unsigned mask) {
+        if constexpr (LOG) {
+            __syncthreads();  // the kSh* words are free from here on
+            float *part = reinterpret_cast<float *>(sh);
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                float v = mt[j];
+#pragma unroll
+                for (int o = 32; o >= 1; o >>= 1) v = v + __shfl_xor(v, o, kWave);
+                if (lane == 0) part[wave * 6 + j] = v;
+            }
+            __syncthreads();
+            if (tid < kMetricSlots && ((mask >> tid) & 1u)) {
+                float v = 0.0f;
+                if (tid < 6)
+                    for (int w = 0; w < kWG / kWave; ++w) v = v + part[w * 6 + tid];
+                P.metrics[(int64_t)item * kMetricSlots + tid] = v;
+            }
+        }
+    }
 
     const FusedParams &P;
     uint32_t *sh, *counter, *hist;
@@ -223,6 +311,10 @@ struct FusedBlock {
         row_in_lds = true;
         holding = false;
         wide = false;
+        if constexpr (LOG) {
+#pragma unroll
+            for (int j = 0; j < 6; ++j) mt[j] = 0.0f;
+        }
     }
 
     __device__ __forceinline__ bool fast_window(const BlockGeo &G) const {
@@ -456,6 +548,10 @@ struct FusedBlock {
             const int off = chunk_off<C>(wave, c, lane);
             float v[8];
             graw[c].to_float(v);
+            if constexpr (LOG) {  // (elements past the block's end were loaded as zeros)
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) log_square(kMtGrad, v[e]);
+            }
             float mn, u;
             if constexpr (kCoop) {
                 const int j0 = c * (kWave / QL);  // first statistic of this chunk in the wave
@@ -561,9 +657,45 @@ struct FusedBlock {
                     for (int j = 0; j < nbytes; ++j)
                         err[(off >> 1) + j] = (uint8_t)(codes >> (8 * j));
                 }
+                if constexpr (LOG || QE) quant_err_chunk(G, c, off, n, x, cf, mnf, u);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+    }
+
+    // What the new error feedback stands for, d = Qinv(e) as a cleared buffer of the
+    // gradient's type receives it (MA:267-268, :321-322): its squares for a logging step, and
+    // with alpha == -2 the parameter steps p = p * decay (MA:234-235), p = p - a (MA:264),
+    // p = p + d (MA:269) on the parameters held in praw, and quant_err = a - d (MA:259-270).
+    __device__ __forceinline__ void quant_err_chunk(const BlockGeo &G, int c, int off, int n,
+                                                    const float (&x)[8], const float (&cf)[8],
+                                                    float mnf, float u) {
+        float pv[8];
+        if constexpr (QE) praw[c].to_float(pv);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            float deq = cf[e] * u;
+            deq = deq + mnf;
+            const float d = to_elem(0.0f + deq);
+            const bool valid = FULL || off + e < n;
+            if (valid) log_square(kMtError, d);
+            if constexpr (QE) {
+                if (G.D.apply_decay != 0) pv[e] = to_elem(pv[e] * G.D.decay);
+                pv[e] = to_elem(pv[e] + (-1.0f) * x[e]);
+                pv[e] = to_elem(pv[e] + d);
+                if (valid) {
+                    const float lost = to_elem(x[e] - d);
+                    log_square(kMtQuantErr, lost);
+                    log_zero(kMtQuantErrZeros, lost);
+                }
+            }
+        }
+        if constexpr (QE) praw[c].from_float(pv);
+    }
+
+    // the weight decay of the update stages: with alpha == -2 it has been applied already
+    __device__ __forceinline__ bool decay_pending(const BlockGeo &G) const {
+        return !QE && G.D.apply_decay != 0;
     }
 
     // ---- Adam direction from the window (MA:277-291), then p = p * (1 - lr*wd) (MA:234-235)
@@ -602,8 +734,8 @@ struct FusedBlock {
                                 // the row (-1 .. kb-1); the row, -1: none
 
     __device__ __forceinline__ bool wide_window(const BlockGeo &G) const {
-        if constexpr (!(R::kBF16 && FULL)) {
-            return false;
+        if constexpr (!(R::kBF16 && FULL) || LOG) {
+            return false;  // (a logging step needs the update of every coordinate)
         } else {
             if (!P.L.compact || !row_in_lds || !fast_window(G)) return false;
             if ((((uintptr_t)G.D.I | (uintptr_t)G.D.V) & 3) != 0) return false;
@@ -802,7 +934,7 @@ struct FusedBlock {
         }
         // nobody reads the cells' marks any more: the last readers passed a barrier above
         const float neg_lr = D.neg_lr;
-        if (D.apply_decay != 0) {
+        if (decay_pending(G)) {
             // every parameter changes: the updates go to the cells, the dense stage does the rest
 #pragma unroll
             for (int j = 0; j < kOwned; ++j)
@@ -844,7 +976,7 @@ struct FusedBlock {
         const TensorDesc &D = G.D;
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
-        const bool apply_decay = D.apply_decay != 0;
+        const bool apply_decay = decay_pending(G);
         WindowView wv;
         wv.I = D.I + G.col0;
         wv.V = D.V + G.col0;
@@ -884,6 +1016,10 @@ struct FusedBlock {
                         if (apply_decay) pv[e] = to_elem(pv[e] * decay);
                         const float prod = neg_lr * u;
                         pv[e] = pv[e] + prod;
+                        if (FULL || off + e < n) {
+                            log_square(kMtUpdate, u);
+                            log_zero(kMtUpdateZeros, u);
+                        }
                     }
                     store8(p, off, FULL ? 0x7fffffff : n, true, pv);
                 }
@@ -1145,7 +1281,7 @@ struct FusedBlock {
         const TensorDesc &D = G.D;
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
-        const bool apply_decay = D.apply_decay != 0;
+        const bool apply_decay = decay_pending(G);
         // the store addresses are formed afresh: kept from the loads, they would sit in
         // registers (or in scratch) through the whole window stage
         const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
@@ -1156,6 +1292,7 @@ struct FusedBlock {
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
                 update8(off, uv);
+                log_update(uv, FULL ? kChunk : n - off);
                 if (apply_decay) {
 #pragma unroll
                     for (int e = 0; e < kChunk; ++e) {
@@ -1237,6 +1374,7 @@ struct FusedBlock {
                 const float u2 = div15(bf2f(mx2b) - m2f, d15);
                 float cf[8];
                 codes8(r2, m2f, u2, cf);
+                log_error(cf, m2f, u2, FULL ? kChunk : n - off);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
                     if (!FULL && off + e >= n) cf[e] = 0.0f;
@@ -1259,7 +1397,7 @@ struct FusedBlock {
         const TensorDesc &D = G.D;
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         const float neg_lr = D.neg_lr, decay = D.decay;
-        const bool apply_decay = D.apply_decay != 0;
+        const bool apply_decay = decay_pending(G);
         // the store addresses are formed afresh: kept from the loads, they would sit in
         // registers (or in scratch) through the whole window stage
         const int tid2 = opaque_tid(), lane2 = tid2 & 63, wave2 = tid2 >> 6;
@@ -1282,6 +1420,10 @@ struct FusedBlock {
                     const float ud = to_elem(uv[e] + add);
                     const float prod = neg_lr * ud;
                     pv[e] = pv[e] + prod;
+                    if (FULL || off + e < n) {
+                        log_square(kMtUpdate, ud);
+                        log_zero(kMtUpdateZeros, ud);
+                    }
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
             }
@@ -1509,6 +1651,10 @@ struct FusedBlock {
             const int off = chunk_off<C>(wave, c, lane);
             float v[8];
             graw[c].to_float(v);
+            if constexpr (LOG) {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) log_square(kMtGrad, v[e]);
+            }
             const bool second = off >= S.bnd;
             const float mn = second ? mn1 : mn0, u = second ? u1 : u0;
 #pragma unroll
@@ -1582,6 +1728,7 @@ struct FusedBlock {
                 float x[8], cf[8];
                 graw[c].to_float(x);
                 codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
+                log_error(cf, second ? mn1 : mn0, second ? u1 : u0, FULL ? kChunk : n - off);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
                     if (!FULL && off + e >= n) cf[e] = 0.0f;
@@ -1620,7 +1767,7 @@ struct FusedBlock {
         elem_t *p = reinterpret_cast<elem_t *>(D.p) + G.e0;
         uint8_t *err = D.err + (G.e0 >> 1);
         const float neg_lr = D.neg_lr, decay = D.decay;
-        const bool apply_decay = D.apply_decay != 0;
+        const bool apply_decay = decay_pending(G);
         const float mn0 = bf2f(sp_mn[0]), mn1 = bf2f(sp_mn[1]);
         const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
         const float m20 = bf2f(sp2_mn[0]), m21 = bf2f(sp2_mn[1]);
@@ -1652,9 +1799,14 @@ struct FusedBlock {
                     pv[e] = pv[e] + prod;
                     const float keep = P.keep * d1[e];
                     r2[e] = to_elem(0.0f + keep);
+                    if (FULL || off + e < n) {
+                        log_square(kMtUpdate, ud);
+                        log_zero(kMtUpdateZeros, ud);
+                    }
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
                 codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
+                log_error(cf, second ? m21 : m20, second ? v1 : v0, FULL ? kChunk : n - off);
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e)
                     if (!FULL && off + e >= n) cf[e] = 0.0f;
@@ -1698,7 +1850,7 @@ __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
 
 // One workgroup per block: any block shape.  Tensor i contributes its blocks
 // blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
-template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false>
+template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false, int AUX = 0>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int item = xcd_contiguous_item(P.total_items);
@@ -1724,12 +1876,13 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
             if constexpr (HOLD) fb.load_held(G, true);
             fb.update(G);
         }
+        fb.log_flush(item, 0xffu);
     };
     if (G.n == R::kC * kRound) {
-        FusedBlock<R, true, QL, HOLD> fb(P, lds);
+        FusedBlock<R, true, QL, HOLD, AUX> fb(P, lds);
         run(fb);
     } else {
-        FusedBlock<R, false, QL, HOLD> fb(P, lds);
+        FusedBlock<R, false, QL, HOLD, AUX> fb(P, lds);
         run(fb);
     }
 }
@@ -1738,7 +1891,9 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
 //   alpha > 0:  PASS 1 (residual and its extremes), PASS 2 (everything else)
 //   alpha == 0: PASS 4 (PASS 1 and the parameter update, which does not wait for the
 //               statistics), PASS 3 (codes of the residual)
-template <class R, int MIN_WAVES, int PASS>
+//   Logging steps: the first pass leaves |g|^2 (and, as PASS 4, the update's sums) and clears
+//   the components no pass forms; the second leaves the rest.
+template <class R, int MIN_WAVES, int PASS, int AUX = 0>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int item = xcd_contiguous_item(P.total_items);
@@ -1768,12 +1923,18 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             fb.template span_statistics<false>(G, S);
             fb.span_codes_stage(G, S);
         }
+        constexpr unsigned kUnused = 1u << kMtQuantErr | 1u << kMtQuantErrZeros | 3u << 6;
+        constexpr unsigned kUpdate = 1u << kMtUpdate | 1u << kMtUpdateZeros;
+        fb.log_flush(item, PASS == 1   ? kUnused | 1u << kMtGrad
+                           : PASS == 4 ? kUnused | 1u << kMtGrad | kUpdate
+                           : PASS == 2 ? kUpdate | 1u << kMtError
+                                       : 1u << kMtError);
     };
     if (G.n == R::kC * kRound) {
-        FusedBlock<R, true, 0> fb(P, lds);
+        FusedBlock<R, true, 0, false, AUX> fb(P, lds);
         run(fb);
     } else {
-        FusedBlock<R, false, 0> fb(P, lds);
+        FusedBlock<R, false, 0, false, AUX> fb(P, lds);
         run(fb);
     }
 }
@@ -1797,17 +1958,30 @@ static int allow_big_lds(K kernel, int bytes) {
 constexpr int kWavesThreeWG = 3 * kWG / 256;  // three workgroups per CU
 constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
-template <class R, int QL, bool DENSE = false, bool HOLD = false>
+template <class R, int QL, bool DENSE = false, bool HOLD = false, int AUX = 0>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // bf16 blocks of up to 20480 elements fit 80 registers and a third of the LDS: three
-    // workgroups per CU; the general window stage with the window held in registers takes the
-    // budget of two
+    // workgroups per CU; the general window stage with the window held in registers, and the
+    // kernels with extras, take the budget of two
     constexpr int kWaves_ =
-        (R::kBF16 && R::kC <= kClass2 && !HOLD) ? kWavesThreeWG : kMinWaves;
-    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD>, lds_bytes);
+        (R::kBF16 && R::kC <= kClass2 && !HOLD && AUX == 0) ? kWavesThreeWG : kMinWaves;
+    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, lds_bytes);
     if (rc) return rc;
-    fused_step_kernel<R, kWaves_, QL, DENSE, HOLD><<<grid, kWG, lds_bytes, s>>>(P);
+    fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX><<<grid, kWG, lds_bytes, s>>>(P);
     return launch_status();
+}
+
+// the kernels with extras (logging, alpha == -2): one per class, any quantisation group
+template <template <int> class RT, bool DENSE, int AUX>
+static int launch_fused_aux(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                            const FusedParams &P) {
+    switch (C) {
+        case kClass0: return launch_fused_one<RT<kClass0>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
 }
 
 // alpha > 0
@@ -1848,43 +2022,44 @@ static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, cons
     return MA_ERR_BLOCK_SIZE;
 }
 
-template <class R>
+template <class R, int AUX = 0>
 static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s,
                            const FusedParams &P) {
     // the first pass has the register needs of the fused kernel
-    constexpr int kFirst = (R::kBF16 && R::kC <= kClass2) ? kWavesThreeWG : kMinWaves;
+    constexpr int kFirst =
+        (R::kBF16 && R::kC <= kClass2 && AUX == 0) ? kWavesThreeWG : kMinWaves;
     int rc;
     switch (pass) {
         case 1:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 1>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 1, AUX>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kFirst, 1><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 1, AUX><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 2:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 2>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 2, AUX>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kFirst, 2><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 2, AUX><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         case 4:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 4>, lds_bytes);
+            rc = allow_big_lds(span_step_kernel<R, kFirst, 4, AUX>, lds_bytes);
             if (rc) return rc;
-            span_step_kernel<R, kFirst, 4><<<grid, kWG, lds_bytes, s>>>(P);
+            span_step_kernel<R, kFirst, 4, AUX><<<grid, kWG, lds_bytes, s>>>(P);
             break;
         default:  // needs the kSh* words only
-            span_step_kernel<R, kMinWaves, 3><<<grid, kWG, kMiscBytes, s>>>(P);
+            span_step_kernel<R, kMinWaves, 3, AUX><<<grid, kWG, kMiscBytes, s>>>(P);
             break;
     }
     return launch_status();
 }
 
-template <template <int> class RT>
+template <template <int> class RT, int AUX = 0>
 static int launch_span(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
                        const FusedParams &P) {
     switch (C) {
-        case kClass0: return launch_span_one<RT<kClass0>>(pass, grid, lds_bytes, s, P);
-        case kClass1: return launch_span_one<RT<kClass1>>(pass, grid, lds_bytes, s, P);
-        case kClass2: return launch_span_one<RT<kClass2>>(pass, grid, lds_bytes, s, P);
-        case kClass3: return launch_span_one<RT<kClass3>>(pass, grid, lds_bytes, s, P);
+        case kClass0: return launch_span_one<RT<kClass0>, AUX>(pass, grid, lds_bytes, s, P);
+        case kClass1: return launch_span_one<RT<kClass1>, AUX>(pass, grid, lds_bytes, s, P);
+        case kClass2: return launch_span_one<RT<kClass2>, AUX>(pass, grid, lds_bytes, s, P);
+        case kClass3: return launch_span_one<RT<kClass3>, AUX>(pass, grid, lds_bytes, s, P);
     }
     return MA_ERR_BLOCK_SIZE;
 }
@@ -1900,5 +2075,18 @@ int launch_span_bf16(int C, int pass, unsigned grid, int lds_bytes, hipStream_t 
                      const FusedParams &P);
 int launch_span_f32(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
                     const FusedParams &P);
+// with extras: aux is a set of kAux* bits, not 0; dense and two-pass steps take kAuxLog only
+int launch_fused_aux_bf16(int C, int aux, unsigned grid, int lds_bytes, hipStream_t s,
+                          const FusedParams &P);
+int launch_fused_aux_f32(int C, int aux, unsigned grid, int lds_bytes, hipStream_t s,
+                         const FusedParams &P);
+int launch_fused_dense_log_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                                const FusedParams &P);
+int launch_fused_dense_log_f32(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                               const FusedParams &P);
+int launch_span_log_bf16(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                         const FusedParams &P);
+int launch_span_log_f32(int C, int pass, unsigned grid, int lds_bytes, hipStream_t s,
+                        const FusedParams &P);
 
 }  // namespace ma

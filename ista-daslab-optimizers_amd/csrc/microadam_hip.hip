@@ -689,10 +689,46 @@ struct PlannedLaunch {
 // blocks of a smaller class ride along in the call's largest class instead.
 constexpr int64_t kMergeBlocks = 768;
 
+// Blocks (work items) a list of tensors makes; -1 for a tensor without elements.
+static int64_t count_blocks(const ma_tensor *tensors, int n_tensors, const ma_hyper *h) {
+    int64_t blocks = 0;
+    for (int i = 0; i < n_tensors; ++i) {
+        if (tensors[i].d <= 0 || h->d_block_size < 1) return -1;
+        const Geometry g = geometry(tensors[i].d, h->d_block_size, h->k_init);
+        blocks += g.n_full + (g.tail > 0 ? 1 : 0);
+    }
+    return blocks;
+}
+
+// Second stage of a logging step's sums: one workgroup adds the blocks' slots in a fixed order,
+// in double, and adds the totals to sums[0..7].
+constexpr int kReduceThreads = 1024;
+__global__ __launch_bounds__(kReduceThreads) void metrics_reduce_kernel(const float *partials,
+                                                                         int64_t blocks,
+                                                                         double *sums) {
+    __shared__ double part[kReduceThreads];
+    // thread t adds component t % 8 of the blocks t / 8, t / 8 + 128, ...
+    const int comp = threadIdx.x % kMetricSlots, first = threadIdx.x / kMetricSlots;
+    double acc = 0.0;
+    for (int64_t b = first; b < blocks; b += kReduceThreads / kMetricSlots)
+        acc += (double)partials[b * kMetricSlots + comp];
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    for (int half = kReduceThreads / 2; half >= kMetricSlots; half >>= 1) {
+        if ((int)threadIdx.x < half) part[threadIdx.x] += part[threadIdx.x + half];
+        __syncthreads();
+    }
+    if (threadIdx.x < kMetricSlots) sums[threadIdx.x] += part[threadIdx.x];
+}
+
+// aux: kAux* bits.  With kAuxLog, metrics holds kMetricSlots floats per block of the call.
 static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h, void *stream,
-                     bool span, double alpha, void *ws, int64_t ws_bytes) {
+                     bool span, double alpha, void *ws, int64_t ws_bytes, int aux = 0,
+                     float *metrics = nullptr) {
     const bool dense = !span && alpha > 0.0;
     if (!tensors || !h || n_tensors < 0) return MA_ERR_ARG;
+    if ((aux & kAuxQuantErr) && (span || dense)) return MA_ERR_NOT_FUSABLE;
+    if ((aux & kAuxLog) && !metrics) return MA_ERR_ARG;
     for (int i = 0; i < n_tensors; ++i) {
         const int rc = span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h);
         if (rc) return rc;
@@ -732,6 +768,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     // ---- all launches are laid out and checked before the first one starts, so that a call
     //      either steps every tensor or none
     std::vector<PlannedLaunch> plan;
+    int64_t items_before = 0;  // work items of the launches laid out so far
     for (int ci = 0; ci < 4; ++ci) {
         int in_class = 0;
         for (int i = 0; i < n_tensors; ++i)
@@ -756,6 +793,8 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.q_span = span ? (int32_t)h->quant_block_size : 0;
             P.alpha = (float)alpha;
             P.keep = (float)(1.0 - alpha);
+            P.metrics = (aux & kAuxLog) ? metrics + items_before * kMetricSlots : nullptr;
+            items_before += items;
             count = 0;
             items = 0;
             dbs_max = kb_max = 0;
@@ -809,17 +848,28 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
         const unsigned grid = (unsigned)P.total_items;
         const bool bf16 = h->dtype == MA_BF16;
         int rc = 0;
-        if (dense) {
+        if (dense && aux) {
+            rc = bf16 ? launch_fused_dense_log_bf16(L.C, grid, P.L.total, s, P)
+                      : launch_fused_dense_log_f32(L.C, grid, P.L.total, s, P);
+        } else if (dense) {
             rc = bf16 ? launch_fused_dense_bf16(L.C, grid, P.L.total, s, P)
                       : launch_fused_dense_f32(L.C, grid, P.L.total, s, P);
+        } else if (!span && aux) {
+            rc = bf16 ? launch_fused_aux_bf16(L.C, aux, grid, P.L.total, s, P)
+                      : launch_fused_aux_f32(L.C, aux, grid, P.L.total, s, P);
         } else if (!span) {
             rc = bf16 ? launch_fused_bf16(L.C, grid, P.L.total, s, P)
                       : launch_fused_f32(L.C, grid, P.L.total, s, P);
         } else {
             const int passes[2] = {alpha > 0.0 ? 1 : 4, alpha > 0.0 ? 2 : 3};
-            for (int i = 0; i < 2 && rc == 0; ++i)
-                rc = bf16 ? launch_span_bf16(L.C, passes[i], grid, P.L.total, s, P)
-                          : launch_span_f32(L.C, passes[i], grid, P.L.total, s, P);
+            for (int i = 0; i < 2 && rc == 0; ++i) {
+                if (aux)
+                    rc = bf16 ? launch_span_log_bf16(L.C, passes[i], grid, P.L.total, s, P)
+                              : launch_span_log_f32(L.C, passes[i], grid, P.L.total, s, P);
+                else
+                    rc = bf16 ? launch_span_bf16(L.C, passes[i], grid, P.L.total, s, P)
+                              : launch_span_f32(L.C, passes[i], grid, P.L.total, s, P);
+            }
         }
         if (rc) return rc;  // the runtime refused a launch: earlier launches of the call stand
     }
@@ -834,6 +884,52 @@ int ma_fused_step_densified(const ma_tensor *tensors, int n_tensors, const ma_hy
                             double alpha, void *stream) {
     if (!(alpha > 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
     return step_impl(tensors, n_tensors, h, stream, false, alpha, nullptr, 0);
+}
+
+int ma_fused_step_quant_err(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
+                            void *stream) {
+    return step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0, kAuxQuantErr);
+}
+
+int64_t ma_logged_step_partials(const ma_tensor *tensors, int n_tensors, const ma_hyper *h) {
+    if (!tensors || !h || n_tensors < 0) return -1;
+    const int64_t blocks = count_blocks(tensors, n_tensors, h);
+    return blocks < 0 ? -1 : blocks * kMetricSlots;
+}
+
+int ma_logged_step(int route, const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
+                   double alpha, void *workspace, int64_t workspace_bytes, float *partials,
+                   int64_t n_partials, double *sums, void *stream) {
+    if (!tensors || !h || n_tensors < 0 || !sums) return MA_ERR_ARG;
+    const int64_t blocks = count_blocks(tensors, n_tensors, h);
+    if (blocks < 0) return MA_ERR_ARG;
+    if (blocks > 0 && (!partials || n_partials < blocks * kMetricSlots ||
+                       ((uintptr_t)partials & 3) != 0))
+        return MA_ERR_ARG;
+    int rc;
+    switch (route) {
+        case MA_ROUTE_FUSED:
+            rc = step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0, kAuxLog, partials);
+            break;
+        case MA_ROUTE_DENSIFIED:
+            if (!(alpha > 0.0) || !(alpha < 1.0)) return MA_ERR_NOT_FUSABLE;
+            rc = step_impl(tensors, n_tensors, h, stream, false, alpha, nullptr, 0, kAuxLog,
+                           partials);
+            break;
+        case MA_ROUTE_SPANNING:
+            rc = step_impl(tensors, n_tensors, h, stream, true, alpha, workspace, workspace_bytes,
+                           kAuxLog, partials);
+            break;
+        case MA_ROUTE_QUANT_ERR:
+            rc = step_impl(tensors, n_tensors, h, stream, false, 0.0, nullptr, 0,
+                           kAuxLog | kAuxQuantErr, partials);
+            break;
+        default:
+            return MA_ERR_ARG;
+    }
+    if (rc || blocks == 0) return rc;
+    metrics_reduce_kernel<<<1, kReduceThreads, 0, (hipStream_t)stream>>>(partials, blocks, sums);
+    return (int)hipGetLastError();
 }
 
 int ma_spanning_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {

@@ -15,6 +15,7 @@ MA_ERR_NOT_FUSABLE = -5
 MA_ERR_LDS = -6
 MA_ERR_WORKSPACE = -7
 MA_STATIC_WORKSPACE_BYTES = 8 << 20
+MA_ROUTE_FUSED, MA_ROUTE_DENSIFIED, MA_ROUTE_SPANNING, MA_ROUTE_QUANT_ERR = 0, 1, 2, 3
 MA_MAX_WINDOW = 64
 
 
@@ -60,6 +61,11 @@ def _load():
         "ma_fused_step_check": (ci, [ctypes.POINTER(MaTensor), ctypes.POINTER(MaHyper)]),
         "ma_fused_step_densified": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
                                          ctypes.c_double, vp]),
+        "ma_fused_step_quant_err": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
+                                         vp]),
+        "ma_logged_step": (ci, [ci, ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
+                                ctypes.c_double, vp, i64, vp, i64, vp, vp]),
+        "ma_logged_step_partials": (i64, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper)]),
         "ma_spanning_step": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
                                    ctypes.c_double, vp, ctypes.c_int64, vp]),
         "ma_spanning_step_static": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
@@ -88,8 +94,10 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_get_max_floats_for_shared_memory_per_thread_block", "ma_copy_values",
            "ma_zerorize_block_components", "ma_asymm_block_quant", "ma_asymm_block_quant_inv",
            "ma_compute_microadam_update", "ma_block_topk", "ma_block_minmax", "ma_param_update",
-           "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified", "ma_spanning_step",
-           "ma_spanning_step_static", "ma_spanning_step_workspace", "ma_spanning_step_check", "ma_sparse_scalar_products",
+           "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified",
+           "ma_fused_step_quant_err", "ma_logged_step", "ma_logged_step_partials",
+           "ma_spanning_step", "ma_spanning_step_static", "ma_spanning_step_workspace",
+           "ma_spanning_step_check", "ma_sparse_scalar_products",
            "ma_sparse_scalar_products_workspace", "ma_sparse_linear_combination",
            "ma_copy_values_typed", "ma_stream_probe")
 

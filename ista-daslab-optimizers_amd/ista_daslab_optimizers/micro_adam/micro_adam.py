@@ -36,7 +36,9 @@ try:  # logging is optional here; the reference imports wandb unconditionally (m
 except Exception:  # pragma: no cover
     wandb = None
 
-OP_BY_OP, FUSED, SPANNING, FUSED_DENSIFIED = 0, 1, 2, 3
+OP_BY_OP, FUSED, SPANNING, FUSED_DENSIFIED, FUSED_QUANT_ERR = 0, 1, 2, 3, 4
+_LOGGED_ROUTE = {FUSED: _hip.MA_ROUTE_FUSED, FUSED_DENSIFIED: _hip.MA_ROUTE_DENSIFIED,
+                 SPANNING: _hip.MA_ROUTE_SPANNING, FUSED_QUANT_ERR: _hip.MA_ROUTE_QUANT_ERR}
 
 # state tensors whose element type the kernels depend on (micro_adam.py:86-94)
 _TYPED_STATE = (('I', torch.int16), ('V', torch.bfloat16), ('error', torch.uint8),
@@ -127,6 +129,7 @@ class MicroAdam(torch.optim.Optimizer):
         self._tables = {}      # (route, dtype) -> _Table
         self._walk = None      # per parameter group: (group, its parameter list, their entries)
         self._workspace = None  # device scratch of the spanning route, grown on demand
+        self._partials = None   # per-block sums of a logging step, grown on demand
 
     # ------------------------------------------------------------------ state (micro_adam.py:61-94)
     def _initialize_parameter_state(self, p, lr, wd):
@@ -199,7 +202,7 @@ class MicroAdam(torch.optim.Optimizer):
         """The route the tensor's sizes and the hyper-parameters admit (the conditions of
         ma_fused_step / ma_spanning_step in include/microadam_hip.h), checked by the library
         itself where it offers the check; what depends on this step's buffers is _fusable's."""
-        if not 0 <= self.alpha < 1 or self.m > _hip.MA_MAX_WINDOW:
+        if not (0 <= self.alpha < 1 or self.alpha == -2) or self.m > _hip.MA_MAX_WINDOW:
             return OP_BY_OP
         # state made for another top-k block size (a checkpoint from other hardware) runs op by
         # op from its stored geometry; the fused kernels derive theirs from self.d_block_size
@@ -216,7 +219,11 @@ class MicroAdam(torch.optim.Optimizer):
         probe.d, probe.k, probe.index = d, st['k'], 0
         h = self._hyper(p.dtype, max(self.steps, 1))
         if _hip.lib.ma_fused_step_check(ctypes.byref(probe), ctypes.byref(h)) == 0:
+            if self.alpha == -2:
+                return FUSED_QUANT_ERR
             return FUSED if self.alpha == 0 else FUSED_DENSIFIED
+        if self.alpha == -2:
+            return OP_BY_OP
         if _hip.lib.ma_spanning_step_check(ctypes.byref(probe), ctypes.byref(h),
                                            float(self.alpha)) == 0:
             return SPANNING
@@ -224,7 +231,7 @@ class MicroAdam(torch.optim.Optimizer):
 
     def _fusable(self, p, st):
         """Route p takes in a step with its current gradient: 0 op by op, 1 fused, 2 spanning,
-        3 fused densified."""
+        3 fused densified, 4 fused with alpha == -2."""
         g = p.grad
         if g.dtype != p.dtype or not p.is_contiguous() or not g.is_contiguous():
             return OP_BY_OP
@@ -260,7 +267,7 @@ class MicroAdam(torch.optim.Optimizer):
         logging_step = self._logging_active() and self.steps % self.log_interval == 0
         totals = dict(norm_qe=0, norm_g=0, norm_u=0, norm_e=0, sparsity_u=0, sparsity_qe=0)
         batches = {}  # (route, dtype) -> entries, in parameter order
-        fused_allowed = self.use_fused and not (logging_step and self.alpha != 0)
+        fused_allowed = self.use_fused
         for group, plist, entries in self._groups():
             lr = group['lr']
             wd = group.get('weight_decay', self.weight_decay)
@@ -272,8 +279,6 @@ class MicroAdam(torch.optim.Optimizer):
                 if e is None or e.st['I'].dtype is not torch.int16:
                     e = entries[i] = self._entry(p, lr, wd)
                 # what this step's buffers admit: same element type, dense, 16-byte aligned
-                # (with alpha != 0 a logging step goes op by op: the update then holds a term
-                # that no state keeps)
                 route = OP_BY_OP
                 if (fused_allowed and e.route and g.dtype is p.dtype and g.is_contiguous()
                         and p.is_contiguous()):
@@ -285,19 +290,20 @@ class MicroAdam(torch.optim.Optimizer):
                         totals[key] += value
                     continue
                 e.lr, e.wd = lr, wd
-                if logging_step:  # before the step: the spanning route overwrites g
-                    totals['norm_g'] += g.view(-1).norm(p=2) ** 2
                 batch = batches.get((route, p.dtype))
                 if batch is None:
                     batch = batches[(route, p.dtype)] = []
                 batch.append(e)
 
+        sums = None  # the fused routes' shares of the logged sums, formed by their kernels
         for (route, dtype), entries in batches.items():
-            self._fused_step(route, dtype, entries)
-            if logging_step:
-                for e in entries:
-                    for key, value in self._metrics_after_fused_step(e.p, e.st).items():
-                        totals[key] += value
+            if logging_step and sums is None:
+                sums = torch.zeros(8, dtype=torch.float64, device=entries[0].p.device)
+            self._fused_step(route, dtype, entries, sums)
+        if sums is not None:
+            for key, value in zip(('norm_qe', 'norm_g', 'norm_u', 'norm_e', 'sparsity_u',
+                                   'sparsity_qe'), sums.tolist()):
+                totals[key] += value
 
         if logging_step:
             self._log(totals['norm_qe'], totals['norm_g'], totals['norm_u'], totals['norm_e'],
@@ -317,28 +323,46 @@ class MicroAdam(torch.optim.Optimizer):
         return walk
 
     # ------------------------------------------------------------------ fused routes
-    def _fused_step(self, route, dtype, entries):
+    def _fused_step(self, route, dtype, entries, sums=None):
+        """One library call for the tensors of one route and element type.  sums: None, or the
+        8 float64 on the device that a logging step's kernels add their sums to
+        (micro_adam.py:155-156, :271-272, :306-308, :320-324)."""
         table = self._tables.get((route, dtype))
         if table is None or len(table.entries) != len(entries) or any(
                 a is not b for a, b in zip(table.entries, entries)):
             table = self._tables[(route, dtype)] = _Table(list(entries))
         table.refresh()
         n, h, stream = len(entries), self._hyper(dtype, self.steps), _hip.stream_ptr()
-        if route == FUSED:
-            rc = _hip.lib.ma_fused_step(table.records, n, ctypes.byref(h), stream)
-            _hip.check(rc, "ma_fused_step")
-        elif route == FUSED_DENSIFIED:
-            rc = _hip.lib.ma_fused_step_densified(table.records, n, ctypes.byref(h),
-                                                  float(self.alpha), stream)
-            _hip.check(rc, "ma_fused_step_densified")
-        else:
+        device = entries[0].p.device
+        alpha, ws_ptr, ws_len = float(self.alpha), None, 0
+        if route == SPANNING:
             need = _hip.lib.ma_spanning_step_workspace(table.records, n, ctypes.byref(h))
-            device = entries[0].p.device
             ws = self._workspace
             if ws is None or ws.numel() < need or ws.device != device:
                 ws = self._workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
-            rc = _hip.lib.ma_spanning_step(table.records, n, ctypes.byref(h), float(self.alpha),
-                                           ws.data_ptr(), ws.numel(), stream)
+            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+        if sums is not None:
+            need = _hip.lib.ma_logged_step_partials(table.records, n, ctypes.byref(h))
+            part = self._partials
+            if part is None or part.numel() < need or part.device != device:
+                part = self._partials = torch.empty(max(need, 8), dtype=torch.float32,
+                                                    device=device)
+            rc = _hip.lib.ma_logged_step(_LOGGED_ROUTE[route], table.records, n, ctypes.byref(h),
+                                         alpha, ws_ptr, ws_len, part.data_ptr(), part.numel(),
+                                         sums.data_ptr(), stream)
+            _hip.check(rc, "ma_logged_step")
+        elif route == FUSED:
+            rc = _hip.lib.ma_fused_step(table.records, n, ctypes.byref(h), stream)
+            _hip.check(rc, "ma_fused_step")
+        elif route == FUSED_DENSIFIED:
+            rc = _hip.lib.ma_fused_step_densified(table.records, n, ctypes.byref(h), alpha, stream)
+            _hip.check(rc, "ma_fused_step_densified")
+        elif route == FUSED_QUANT_ERR:
+            rc = _hip.lib.ma_fused_step_quant_err(table.records, n, ctypes.byref(h), stream)
+            _hip.check(rc, "ma_fused_step_quant_err")
+        else:
+            rc = _hip.lib.ma_spanning_step(table.records, n, ctypes.byref(h), alpha, ws_ptr,
+                                           ws_len, stream)
             _hip.check(rc, "ma_spanning_step")
         for e in entries:  # micro_adam.py:211
             e.st['index'] = (e.st['index'] + 1) % self.m
@@ -431,25 +455,6 @@ class MicroAdam(torch.optim.Optimizer):
             acc.zero_()
             add_dequantised(1.0)
             out['norm_e'] = acc.norm(p=2) ** 2
-        return out
-
-    def _metrics_after_fused_step(self, p, st):
-        """norm_u, norm_e and the update's zero count (micro_adam.py:306-308, :320-324) for a
-        tensor that a fused kernel has just stepped with alpha == 0: the update is rebuilt from
-        the window (which already holds this step's row, as at micro_adam.py:277-291) and the
-        error norm from the stored error feedback, both in p.grad, which the step leaves as
-        scratch like the reference does (:276, :321)."""
-        scratch = p.grad.view(-1)
-        scratch.zero_()
-        _ext_quant.compute_microadam_update(st['blocks'], self.threads, self.shared_memory_carveout,
-                                            self.steps, self.beta1, self.beta2, self.eps,
-                                            st['d_block_size'], st['k_block_size_many'], st['d'],
-                                            self.m, st['k'], st['I'], st['V'], scratch)
-        out = dict(norm_u=scratch.norm(p=2) ** 2, sparsity_u=(scratch == 0).sum())
-        scratch.zero_()
-        _ext_quant.asymm_block_quant_inv(st['d'], self.quant_block_size, st['error'], st['min_vals'],
-                                         st['max_vals'], scratch, 1.0)
-        out['norm_e'] = scratch.norm(p=2) ** 2
         return out
 
     # ------------------------------------------------------------------ checkpointing

@@ -391,12 +391,36 @@ typedef struct {
 /* micro_adam.py:146-328 for alpha in [0, 1) and alpha == -2.  `grad` is consumed as scratch, as in
  * the reference (:153).  `index` is the ring position (:180, :211) and is
  * advanced.  Returns 0, or -1 for any other alpha. */
-int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d, int64_t *index,
-                    int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
-                    uint16_t *max_vals) {
+static double sum_squares(const void *x, int64_t d, int dtype) {
+    double s = 0;
+    for (int64_t i = 0; i < d; ++i) {
+        const double v = ld(x, i, dtype);
+        s += v * v;
+    }
+    return s;
+}
+
+static double count_zeros(const void *x, int64_t d, int dtype) {
+    int64_t n = 0;
+    for (int64_t i = 0; i < d; ++i) n += ld(x, i, dtype) == 0.0f;
+    return (double)n;
+}
+
+static void clear(void *x, int64_t d, int dtype) {
+    memset(x, 0, (size_t)d * (dtype == ORA_BF16 ? 2 : 4));
+}
+
+/* mt: NULL, or the six sums a logging step adds up over the tensors (micro_adam.py:148, :328):
+ * [0] |quant_err|^2 (:271), [1] |g|^2 (:155-156), [2] |u|^2 (:307), [3] |Qinv(e)|^2 (:320-324),
+ * [4] zeros of u (:308), [5] zeros of quant_err (:272); each += this tensor's share, taken in
+ * double from the values as the buffer holds them (rounded to the gradient's type). */
+static int update_step_impl(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d,
+                            int64_t *index, int16_t *I, uint16_t *V, uint8_t *error,
+                            uint16_t *min_vals, uint16_t *max_vals, double *mt) {
     ora_geom g;
     if (h->alpha < 0 && h->alpha != -2.0) return -1;
     ora_geometry(d, h->max_d_block_size, h->k_init, h->q, &g);
+    if (mt) mt[1] += sum_squares(grad, d, dtype);
     int64_t row = *index;
     int16_t *I_row = I + row * g.k;
     uint16_t *V_row = V + row * g.k;
@@ -420,15 +444,25 @@ int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t 
     /* :238-273, alpha == -2: p = p - a + Qinv(e_new).  The quant_err vector of :259-261, :271
      * only feeds the logged norms. */
     if (h->alpha == -2.0) {
+        void *qe = NULL;
+        if (mt) { /* :259-261: quant_err = a (it has the parameter's type) */
+            qe = malloc((size_t)d * 4);
+            if (!qe) return -2;
+            memcpy(qe, grad, (size_t)d * (dtype == ORA_BF16 ? 2 : 4));
+        }
         ora_param_update(d, p, grad, -1.0f, dtype, dtype);                       /* STEP A, :264 */
-        if (dtype == ORA_BF16) memset(grad, 0, (size_t)d * 2);                   /* :267 */
-        else memset(grad, 0, (size_t)d * 4);
+        clear(grad, d, dtype);                                                   /* :267 */
         ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad, 1.0f, dtype);
         ora_param_update(d, p, grad, 1.0f, dtype, dtype);                        /* STEP B, :269 */
+        if (mt) { /* :271-273: quant_err -= Qinv(e_new), rounded to its type */
+            for (int64_t i = 0; i < d; ++i) st(qe, i, dtype, ld(qe, i, dtype) - ld(grad, i, dtype));
+            mt[0] += sum_squares(qe, d, dtype);
+            mt[5] += count_zeros(qe, d, dtype);
+            free(qe);
+        }
     }
     /* STEPS 10-11, :276-291 */
-    if (dtype == ORA_BF16) memset(grad, 0, (size_t)d * 2);
-    else memset(grad, 0, (size_t)d * 4);
+    clear(grad, d, dtype);
     ora_compute_microadam_update(h->t, h->beta1, h->beta2, h->eps, g.d_block_size,
                                  g.k_block_size_many, d, h->m, g.k, I, V, grad, dtype);
     /* :296-298 */
@@ -436,16 +470,40 @@ int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t 
         ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad, (float)h->alpha, dtype);
     /* STEP 12, :304 */
     ora_param_update(d, p, grad, (float)(-h->lr), dtype, dtype);
+    if (mt) { /* :306-308 */
+        mt[2] += sum_squares(grad, d, dtype);
+        mt[4] += count_zeros(grad, d, dtype);
+    }
     /* :311-316 */
     if (h->alpha > 0) {
-        if (dtype == ORA_BF16) memset(grad, 0, (size_t)d * 2);
-        else memset(grad, 0, (size_t)d * 4);
+        clear(grad, d, dtype);
         ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad,
                                   (float)(1.0 - h->alpha), dtype);
         ora_block_minmax(d, h->q, grad, dtype, min_vals, max_vals);
         ora_asymm_block_quant(d, h->q, error, min_vals, max_vals, grad, dtype);
     }
+    if (mt) { /* :320-324 */
+        clear(grad, d, dtype);
+        ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad, 1.0f, dtype);
+        mt[3] += sum_squares(grad, d, dtype);
+    }
     return 0;
+}
+
+int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d, int64_t *index,
+                    int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
+                    uint16_t *max_vals) {
+    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, NULL);
+}
+
+/* A logging step (micro_adam.py:155-156, :271-272, :306-308, :320-324): ora_update_step, and
+ * the tensor's shares added to metrics[0..5] = norm_qe, norm_g, norm_u, norm_e, sp_u, sp_qe
+ * (the order of the reference's return value, :328; squared norms, counts of zeros). */
+int ora_step_metrics(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d, int64_t *index,
+                     int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
+                     uint16_t *max_vals, double *metrics) {
+    if (!metrics) return -1;
+    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, metrics);
 }
 
 /* ---- Sparse M-FAC's two window kernels (same I / V layout) ---------------- */

@@ -76,6 +76,8 @@ def lib():
         L.ora_update_step.argtypes = [ctypes.POINTER(_Hyper), vp, vp, ci, i64,
                                       ctypes.POINTER(i64), vp, vp, vp, vp, vp]
         L.ora_update_step.restype = ci
+        L.ora_step_metrics.argtypes = L.ora_update_step.argtypes + [ctypes.POINTER(f64)]
+        L.ora_step_metrics.restype = ci
         L.ora_sparse_scalar_products.argtypes = [i64, i64, i64, i64, i64, vp, ci, vp, vp, ci, vp]
         L.ora_sparse_linear_combination.argtypes = [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp,
                                                     ci]
@@ -252,11 +254,17 @@ class OracleMicroAdam:
         self.state[i] = st
         return st
 
-    def step(self, grads, lr=None):
+    METRICS = ("norm_qe", "norm_g", "norm_u", "norm_e", "sparsity_u", "sparsity_qe")
+
+    def step(self, grads, lr=None, metrics=False):
+        """One optimizer step.  metrics=True: a logging step (micro_adam.py:155-156, :271-272,
+        :306-308, :320-324); returns the six sums over the tensors that the reference hands
+        to its _log (:328, :330) as a dict of Python floats: squared norms and zero counts."""
         self.steps += 1
         lr = self.lr if lr is None else lr
         h = _Hyper(self.steps, self.m, self.quant_block_size, self.d_block_size, self.k_init,
                    float(self.alpha), self.beta1, self.beta2, self.eps, lr, self.weight_decay)
+        sums = (ctypes.c_double * 6)()
         for i, (p, g) in enumerate(zip(self.params, grads)):
             if g is None:
                 continue
@@ -264,10 +272,11 @@ class OracleMicroAdam:
             assert g.dtype == p.dtype and g.size == p.size
             st = self.state[i] or self._init_state(i)
             idx = ctypes.c_int64(st["index"])
-            rc = lib().ora_update_step(ctypes.byref(h), _ptr(p), _ptr(g), dtype_tag(p), p.size,
-                                       ctypes.byref(idx), _ptr(st["I"]), _ptr(st["V"]),
-                                       _ptr(st["error"]), _ptr(st["min_vals"]),
-                                       _ptr(st["max_vals"]))
+            args = (ctypes.byref(h), _ptr(p), _ptr(g), dtype_tag(p), p.size, ctypes.byref(idx),
+                    _ptr(st["I"]), _ptr(st["V"]), _ptr(st["error"]), _ptr(st["min_vals"]),
+                    _ptr(st["max_vals"]))
+            rc = lib().ora_step_metrics(*args, sums) if metrics else lib().ora_update_step(*args)
             if rc != 0:
                 raise NotImplementedError("oracle covers alpha in [0, 1) and alpha == -2")
             st["index"] = idx.value
+        return dict(zip(self.METRICS, sums)) if metrics else None

@@ -431,6 +431,51 @@ def test_whole_step_matches_torch_restatement(oracle, sizes, dtype, m, q, k_init
             assert np.array_equal(bits(tref.params[i]), oparams[i]), (s, i)
 
 
+@pytest.mark.parametrize("sizes,dtype,m,q,k_init,alpha,wd,DB,steps", CASES)
+def test_logged_sums_match_torch_restatement(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB,
+                                             steps):
+    """The six sums of a logging step (micro_adam.py:155-156, :271-272, :306-308, :320-324)
+    against the same sums taken with torch at the same points of the restated step.  Both sum
+    the same values in float64; only the order of the additions differs (1e-12 relative).
+    Placement matters and is what this pins: |u|^2 includes alpha * Qinv(e), the error norm is
+    of the error feedback after the step's last requantisation, |g|^2 of the untouched
+    gradient."""
+    gen = torch.Generator().manual_seed(1)
+    params = [(torch.randn(n, generator=gen) * 0.02).to(dtype) for n in sizes]
+    tref = TorchMicroAdam([p.clone() for p in params], m, 1e-3, q, k_init, alpha,
+                          weight_decay=wd, d_block_size=DB)
+    oref = oracle.OracleMicroAdam([bits(p) for p in params], m, 1e-3, q, k_init, alpha,
+                                  weight_decay=wd, d_block_size=DB)
+    seen_nonzero = set()
+    for s in range(steps):
+        grads = [(torch.randn(n, generator=gen) * 0.01).to(dtype) for n in sizes]
+        want = tref.step([g.clone() for g in grads], metrics=True)
+        got = oref.step([bits(g) for g in grads], metrics=True)
+        assert set(got) == set(want)
+        for key in want:
+            assert got[key] == pytest.approx(want[key], rel=1e-12, abs=0), (s, key)
+            if want[key] != 0:
+                seen_nonzero.add(key)
+    expect = {"norm_g", "norm_u", "norm_e"}
+    if alpha <= 0:
+        expect |= {"sparsity_u"}  # (alpha > 0 makes the update dense)
+    if alpha == -2:
+        expect |= {"norm_qe"}
+    assert expect <= seen_nonzero
+    # a step without metrics moves the state exactly as one with them
+    a = oracle.OracleMicroAdam([bits(p) for p in params], m, 1e-3, q, k_init, alpha,
+                               weight_decay=wd, d_block_size=DB)
+    b = oracle.OracleMicroAdam([bits(p) for p in params], m, 1e-3, q, k_init, alpha,
+                               weight_decay=wd, d_block_size=DB)
+    for s in range(3):
+        grads = [bits((torch.randn(n, generator=gen) * 0.01).to(dtype)) for n in sizes]
+        assert a.step([g.copy() for g in grads]) is None
+        b.step([g.copy() for g in grads], metrics=True)
+        for i in range(len(sizes)):
+            assert np.array_equal(a.params[i], b.params[i])
+            assert np.array_equal(a.state[i]["error"], b.state[i]["error"])
+
+
 def test_error_feedback_invariant(oracle):
     """a_t = g_t + Qinv(e_t); after the step Qinv(e_{t+1}) reproduces a_t with the top-k
     entries removed, to within half a quantisation step."""

@@ -127,14 +127,23 @@ class TorchMicroAdam:
         out = (z1 * s1) / (torch.tensor(self.eps, dtype=torch.float32) + root)
         grad[hit] = out[hit].to(grad.dtype)
 
-    def step(self, grads, lr=None):
+    def step(self, grads, lr=None, metrics=False):
+        """metrics=True: also the sums of a logging step, taken with torch at the points of
+        micro_adam.py:155-156, :258-273, :306-308, :320-324 (in float64, from the buffers as they
+        are at that point)."""
         self.steps += 1
         lr = self.lr if lr is None else lr
+        sums = dict(norm_qe=0.0, norm_g=0.0, norm_u=0.0, norm_e=0.0, sparsity_u=0.0, sparsity_qe=0.0)
+
+        def sq(x):
+            return float(x.double().pow(2).sum())
+
         for i, (p, grad) in enumerate(zip(self.params, grads)):
             if grad is None:
                 continue
             grad = grad.view(-1)
             d = p.numel()
+            sums["norm_g"] += sq(grad)
             st = self.state[i] or self._init(i)
             index, I, V = st["index"], st["I"], st["V"]
             dbs, full, dit = st["dbs"], st["full"], st["d_index_topk"]
@@ -154,20 +163,32 @@ class TorchMicroAdam:
             if self.wd > 0:
                 p.mul_(1 - lr * self.wd)
             if self.alpha == -2:
-                # micro_adam.py:264-269: p = p - a, then p = p + Qinv(e_new)
+                # micro_adam.py:258-273: p = p - a, then p = p + Qinv(e_new); quant_err = a - Qinv(e_new)
+                quant_err = torch.zeros_like(p).view(-1)
+                quant_err.add_(grad)
                 p.add_(grad, alpha=-1)
                 grad.zero_()
                 qinv_accumulate(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad, 1.0)
                 p.add_(grad)
+                quant_err.sub_(grad)
+                sums["norm_qe"] += sq(quant_err)
+                sums["sparsity_qe"] += float((quant_err == 0).sum())
             grad.zero_()
             self._adam_direction(st, grad, d)
             if self.alpha > 0:
                 qinv_accumulate(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad,
                                 self.alpha)
             p.copy_((p.float() + torch.tensor(-lr, dtype=torch.float32) * grad.float()).to(p.dtype))
+            sums["norm_u"] += sq(grad)
+            sums["sparsity_u"] += float((grad == 0).sum())
             if self.alpha > 0:
                 grad.zero_()
                 qinv_accumulate(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad,
                                 1 - self.alpha)
                 self._stats(st, grad, d)
                 quantize(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad)
+            if metrics:
+                grad.zero_()
+                qinv_accumulate(d, self.q, st["error"], st["min_vals"], st["max_vals"], grad, 1.0)
+                sums["norm_e"] += sq(grad)
+        return sums if metrics else None
