@@ -269,6 +269,78 @@ def test_state_layout_and_checkpoint_roundtrip():
     assert torch.equal(p.data, p2.data)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_checkpoint_through_a_file(oracle, tmp_path, dtype):
+    """torch.save -> torch.load(weights_only=True) -> load_state_dict into a fresh optimizer,
+    mid-run and after the ring has wrapped: the resumed run continues bit for bit like the
+    uninterrupted one and like the oracle (which never stopped), on the fused route."""
+    from ista_daslab_optimizers import MicroAdam
+    sizes, m = [20480 * 2 + 4096, 768], 4
+    gen = torch.Generator().manual_seed(5)
+    cpu_params = [(torch.randn(n, generator=gen) * 0.02).to(dtype) for n in sizes]
+    oparams = [to_np(p) for p in cpu_params]
+    oref = oracle.OracleMicroAdam(oparams, m, 1e-3, 64, 0.01, 0, weight_decay=0.01)
+    params = [torch.nn.Parameter(p.clone().cuda()) for p in cpu_params]
+    opt = MicroAdam(params, m=m, lr=1e-3, quant_block_size=64, weight_decay=0.01)
+    for s in range(11):
+        if s in (2, 7):  # before and after the window is full
+            path = tmp_path / f"ckpt{s}.pt"
+            torch.save({"opt": opt.state_dict(), "params": [p.data for p in params]}, path)
+            del opt, params
+            blob = torch.load(path, map_location="cuda", weights_only=True)
+            params = [torch.nn.Parameter(t.clone()) for t in blob["params"]]
+            opt = MicroAdam(params, m=m, lr=1e-3, quant_block_size=64, weight_decay=0.01)
+            opt.load_state_dict(blob["opt"])
+            assert opt.steps == s
+            for p in params:
+                st = opt.state[p]
+                assert st["I"].dtype == torch.int16 and st["error"].dtype == torch.uint8
+                assert st["V"].dtype == st["min_vals"].dtype == torch.bfloat16
+                assert st["index"] == s % m
+        grads = [(torch.randn(n, generator=gen) * 1e-2).to(dtype) for n in sizes]
+        for p, g in zip(params, grads):
+            p.grad = g.clone().cuda()
+        opt.step()
+        assert all(opt._fusable(p, opt.state[p]) == 1 for p in params)
+        oref.step([to_np(g) for g in grads])
+        for i, p in enumerate(params):
+            assert_state_equal(opt.state[p], oref.state[i], f"step {s + 1} tensor {i}")
+            assert np.array_equal(to_np(p.data), oparams[i]), f"step {s + 1} tensor {i}"
+
+
+def test_checkpoint_made_for_another_block_size(oracle):
+    """State whose geometry was derived from another device's top-k block size (the reference
+    sizes d_block_size from the shared memory of the GPU it runs on, micro_adam.py:43-44): the
+    fused kernels would derive a different geometry from this optimizer's own, so such tensors
+    take the op-by-op route, which reads the stored geometry, and still match an oracle that
+    runs with the checkpoint's block size."""
+    from ista_daslab_optimizers import MicroAdam
+    n, m, foreign = 20480 * 2 + 4096, 4, 12288
+    gen = torch.Generator().manual_seed(6)
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(torch.bfloat16)
+    oparams = [to_np(p0)]
+    oref = oracle.OracleMicroAdam(oparams, m, 1e-3, 64, 0.01, 0, d_block_size=foreign)
+    p = torch.nn.Parameter(p0.clone().cuda())
+    src = MicroAdam([p], m=m, lr=1e-3, quant_block_size=64)
+    src.d_block_size = foreign
+    grads = [(torch.randn(n, generator=gen) * 1e-2).to(torch.bfloat16) for _ in range(6)]
+    for g in grads[:3]:
+        p.grad = g.clone().cuda()
+        src.step()
+        oref.step([to_np(g)])
+    assert src.state[p]["d_block_size"] == foreign
+    p2 = torch.nn.Parameter(p.detach().clone())
+    dst = MicroAdam([p2], m=m, lr=1e-3, quant_block_size=64)   # d_block_size 20480
+    dst.load_state_dict(src.state_dict())
+    for s, g in enumerate(grads[3:]):
+        p2.grad = g.clone().cuda()
+        dst.step()
+        assert dst._fusable(p2, dst.state[p2]) == 0
+        oref.step([to_np(g)])
+        assert_state_equal(dst.state[p2], oref.state[0], f"resumed step {s + 1}")
+        assert np.array_equal(to_np(p2.data), oparams[0]), f"resumed step {s + 1}"
+
+
 def test_cpu_parameter_is_rejected():
     from ista_daslab_optimizers import MicroAdam
     p = torch.nn.Parameter(torch.zeros(100))
