@@ -486,14 +486,14 @@ def test_quantisation_rounding_boundaries(oracle, dtype, use_fused):
     """The 4-bit codes where they are hardest to get right: every quantisation block holds its
     minimum 0, its maximum M, and for each of the 15 rounding boundaries the value nearest to
     (k + 1/2) u and its two neighbours (u = (M - 0) / 15 as the kernels form it), with M running
-    through bf16 significands and through binary exponents -120 .. 120, so that steps u that are
-    tiny, ordinary and huge all occur.  The fused kernels divide by a shared reciprocal where the
+    through bf16 significands and through every binary exponent from -126 to 126, so that steps u
+    that are subnormal, tiny, ordinary and huge all occur.  The fused kernels divide by a shared reciprocal where the
     oracle divides; the codes must agree bit for bit all the same.  A second step with a zero
     gradient dequantises and requantises them."""
     from ista_daslab_optimizers import MicroAdam
     q, DB = 64, 4096
     sig = [1.0, 1.0078125, 1.25, 1.5, 1.9921875, 1.328125, 1.7109375]
-    exps = list(range(-120, 121, 5))
+    exps = list(range(-126, 127))
     gen = torch.Generator().manual_seed(17)
     blocks = []
     for e in exps:
