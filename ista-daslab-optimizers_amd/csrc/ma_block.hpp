@@ -787,9 +787,24 @@ struct FusedBlock {
     }
 
     __device__ __forceinline__ void update_wide(const BlockGeo &G) {
-        if constexpr (R::kBF16 && FULL) update_wide_bf16(G);
+        if constexpr (R::kBF16 && FULL) update_wide_bf16<false>(G);
     }
 
+    // The window stage alone: the slot cells end up holding the update's bits (0 where no
+    // window row names the coordinate), for a parameter stage of the caller's.  Ends with a
+    // barrier.
+    __device__ __forceinline__ void window_cells(const BlockGeo &G) {
+        if constexpr (R::kBF16 && FULL) {
+            if (wide) {
+                update_wide_bf16<true>(G);
+                return;
+            }
+        }
+        window_stage(G);
+    }
+
+    // CELLS_ONLY: stop once the cells hold the updates (window_cells)
+    template <bool CELLS_ONLY>
     __device__ __forceinline__ void update_wide_bf16(const BlockGeo &G) {
         constexpr int n = C * kRound;
         constexpr int kSlots = 5;  // four entries of an older row, one of this step's row
@@ -883,7 +898,7 @@ struct FusedBlock {
             slot_clear = false;
             load_window(G);
             window_stage(G);
-            param_stage(G);
+            if (!CELLS_ONLY) param_stage(G);
             return;
         }
         if (queued != 0) {
@@ -934,13 +949,13 @@ struct FusedBlock {
         }
         // nobody reads the cells' marks any more: the last readers passed a barrier above
         const float neg_lr = D.neg_lr;
-        if (decay_pending(G)) {
+        if (CELLS_ONLY || decay_pending(G)) {
             // every parameter changes: the updates go to the cells, the dense stage does the rest
 #pragma unroll
             for (int j = 0; j < kOwned; ++j)
                 if (upd[j] != 0xffffffffu) cell16[upd[j] & 0xffffu] = (uint16_t)(upd[j] >> 16);
             __syncthreads();
-            param_stage(G);
+            if (!CELLS_ONLY) param_stage(G);
             return;
         }
 #pragma unroll
@@ -1706,6 +1721,33 @@ struct FusedBlock {
     }
 
     // ---- pass 2 -----------------------------------------------------------------------
+    // The window row the first pass wrote comes back into sel_idx / sel_val, where the window
+    // stages expect the row of this step: requested first, stored once the other requests
+    // are out.
+    uint32_t row_i, row_v;
+
+    __device__ __forceinline__ void span_load_row(const BlockGeo &G) {
+        row_i = row_v = 0;
+        if (tid < G.kb) {
+            const int64_t at = (int64_t)G.D.row * G.D.k + G.col0 + tid;
+            row_i = reinterpret_cast<const uint16_t *>(G.D.I)[at];
+            row_v = G.D.V[at];
+        }
+        row_in_lds = true;
+    }
+
+    __device__ __forceinline__ void span_row_to_lds(const BlockGeo &G) {
+        if (tid < G.kb) {
+            sel_idx[tid] = (uint16_t)row_i;
+            sel_val[tid] = (uint16_t)row_v;
+        }
+        for (int j = tid + kWG; j < G.kb; j += kWG) {
+            const int64_t at = (int64_t)G.D.row * G.D.k + G.col0 + j;
+            sel_idx[j] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
+            sel_val[j] = G.D.V[at];
+        }
+    }
+
     __device__ __forceinline__ void span_load_residual(const BlockGeo &G) {
         const int n = FULL ? C * kRound : G.n;
         const elem_t *g = reinterpret_cast<const elem_t *>(G.D.g) + G.e0;
@@ -1760,7 +1802,10 @@ struct FusedBlock {
     }
 
     // alpha > 0, second pass: p = p * decay; u = rne(Adam + alpha * d1); p += -lr * u;
-    // r2 = rne(0 + keep * d1); e = Q(r2); the statistics arrays.  After window_stage.
+    // r2 = rne(0 + keep * d1); e = Q(r2); the statistics arrays.  After window_cells.
+    // d1 = Qinv(e1) takes 16 values per segment, and alpha * d1 and the code of r2 with them:
+    // both come from a table of 2 x 16 entries that 32 threads fill first, so that an element
+    // costs one quantisation, not two.
     __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
@@ -1772,45 +1817,59 @@ struct FusedBlock {
         const float u0 = div15(bf2f(sp_mx[0]) - mn0, d15), u1 = div15(bf2f(sp_mx[1]) - mn1, d15);
         const float m20 = bf2f(sp2_mn[0]), m21 = bf2f(sp2_mn[1]);
         const float v0 = div15(bf2f(sp2_mx[0]) - m20, d15), v1 = div15(bf2f(sp2_mx[1]) - m21, d15);
+        // [segment][code]: alpha * d1, code of r2; in the kSh* words, which the window stage
+        // has finished with (the fp32 window stage leaves the updates in its own arrays)
+        static_assert(kMiscBytes >= 32 * 8, "the table takes the kSh* words");
+        uint2 *table = reinterpret_cast<uint2 *>(sh);
+        if (tid < 32) {
+            const bool second = tid >= 16;
+            const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
+            float deq = (float)(tid & 15) * u;
+            const float d1 = deq + mnf;
+            const float add = P.alpha * d1;
+            const float keep = P.keep * d1;
+            float r2[8], c2[8];
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) r2[e] = to_elem(0.0f + keep);
+            codes8(r2, second ? m21 : m20, second ? v1 : v0, c2);
+            table[tid] = make_uint2(__float_as_uint(add), (uint32_t)c2[0]);
+        }
+        __syncthreads();
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
             if (FULL || off < n) {
                 const bool second = off >= S.bnd;
-                float x[8], cf[8], d1[8];
+                float x[8], cf[8];
                 graw[c].to_float(x);
                 codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
-                const float mnf = second ? mn1 : mn0, u = second ? u1 : u0;
-#pragma unroll
-                for (int e = 0; e < kChunk; ++e) {
-                    float deq = cf[e] * u;
-                    d1[e] = deq + mnf;
-                }
+                const uint2 *mine = table + (second ? 16 : 0);
                 float pv[8], uv[8];
                 praw[c].to_float(pv);
                 update8(off, uv);
-                float r2[8];
+                uint32_t codes = 0;
 #pragma unroll
                 for (int e = 0; e < kChunk; ++e) {
+                    const uint2 t = mine[(uint32_t)cf[e]];
                     if (apply_decay) pv[e] = to_elem(pv[e] * decay);
-                    const float add = P.alpha * d1[e];
-                    const float ud = to_elem(uv[e] + add);
+                    const float ud = to_elem(uv[e] + __uint_as_float(t.x));
                     const float prod = neg_lr * ud;
                     pv[e] = pv[e] + prod;
-                    const float keep = P.keep * d1[e];
-                    r2[e] = to_elem(0.0f + keep);
-                    if (FULL || off + e < n) {
-                        log_square(kMtUpdate, ud);
-                        log_zero(kMtUpdateZeros, ud);
+                    const bool valid = FULL || off + e < n;
+                    // nibble order (e0 e1)(e2 e3) | (e4 e5)(e6 e7), even element high
+                    constexpr int kShift[8] = {4, 0, 12, 8, 20, 16, 28, 24};
+                    if (valid) codes |= t.y << kShift[e];
+                    if constexpr (LOG) {
+                        if (valid) {
+                            log_square(kMtUpdate, ud);
+                            log_zero(kMtUpdateZeros, ud);
+                            float deq = (float)t.y * (second ? v1 : v0);
+                            deq = deq + (second ? m21 : m20);
+                            log_square(kMtError, to_elem(0.0f + deq));
+                        }
                     }
                 }
                 store8(p, off, FULL ? 0x7fffffff : n, true, pv);
-                codes8(r2, second ? m21 : m20, second ? v1 : v0, cf);
-                log_error(cf, second ? m21 : m20, second ? v1 : v0, FULL ? kChunk : n - off);
-#pragma unroll
-                for (int e = 0; e < kChunk; ++e)
-                    if (!FULL && off + e >= n) cf[e] = 0.0f;
-                const uint32_t codes = pack_codes(cf);
                 if (FULL || off + kChunk <= n) {
                     *reinterpret_cast<uint32_t *>(err + ((unsigned)off >> 1)) = codes;
                 } else {
@@ -1911,12 +1970,14 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
                 fb.update(G);
             }
         } else if constexpr (PASS == 2) {
-            fb.row_in_lds = false;
-            fb.load_window(G);
-            fb.span_load_residual(G);
+            fb.span_load_row(G);
+            fb.load_params_window(G);
+            fb.span_row_to_lds(G);
             fb.template span_statistics<true>(G, S);
-            fb.load_params(G);
-            fb.window_stage(G);
+            fb.window_cells(G);
+            // (asked for only now: held through the window stage, the residual would cost
+            // the registers that stage needs)
+            fb.span_load_residual(G);
             fb.span_param_stage(G, S);
         } else {
             fb.span_load_residual(G);
