@@ -627,11 +627,16 @@ struct FusedBlock {
             float x[8];
             float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < kChunk; ++e) {
-                x[e] = r.val(c, e);
-                if (FULL || off + e < n) {
-                    mn = fmin_raw(mn, x[e]);
-                    mx = fmax_raw(mx, x[e]);
+            for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+            if (FULL) {
+                minmax8(x, mn, mx);
+            } else {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (off + e < n) {
+                        mn = fmin_raw(mn, x[e]);
+                        mx = fmax_raw(mx, x[e]);
+                    }
                 }
             }
             group_minmax<QL>(mn, mx, ql);
@@ -1343,11 +1348,16 @@ struct FusedBlock {
             float x[8];
             float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < kChunk; ++e) {
-                x[e] = r.val(c, e);
-                if (FULL || off + e < n) {
-                    mn = fmin_raw(mn, x[e]);
-                    mx = fmax_raw(mx, x[e]);
+            for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+            if (FULL) {
+                minmax8(x, mn, mx);
+            } else {
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (off + e < n) {
+                        mn = fmin_raw(mn, x[e]);
+                        mx = fmax_raw(mx, x[e]);
+                    }
                 }
             }
             group_minmax<QL>(mn, mx, ql);
@@ -1702,11 +1712,16 @@ struct FusedBlock {
                 float x[8];
                 float lmn = INFINITY, lmx = -INFINITY;
 #pragma unroll
-                for (int e = 0; e < kChunk; ++e) {
-                    x[e] = r.val(c, e);
-                    if (FULL || off + e < n) {
-                        lmn = fmin_raw(lmn, x[e]);
-                        lmx = fmax_raw(lmx, x[e]);
+                for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+                if (FULL) {
+                    minmax8(x, lmn, lmx);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        if (off + e < n) {
+                            lmn = fmin_raw(lmn, x[e]);
+                            lmx = fmax_raw(lmx, x[e]);
+                        }
                     }
                 }
                 const bool second = off >= S.bnd;

@@ -101,6 +101,23 @@ __device__ __forceinline__ float fmax_raw(float a, float b) {
     return d;
 }
 
+// the same of three numbers, still one instruction
+__device__ __forceinline__ float fmin3_raw(float a, float b, float c) {
+    float d;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+__device__ __forceinline__ float fmax3_raw(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+// min and max of the 8 values of a chunk: four instructions each
+__device__ __forceinline__ void minmax8(const float (&x)[8], float &mn, float &mx) {
+    mn = fmin_raw(fmin3_raw(fmin3_raw(fmin3_raw(x[0], x[1], x[2]), x[3], x[4]), x[5], x[6]), x[7]);
+    mx = fmax_raw(fmax3_raw(fmax3_raw(fmax3_raw(x[0], x[1], x[2]), x[3], x[4]), x[5], x[6]), x[7]);
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_perm(float v) {
     return __int_as_float(
