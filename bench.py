@@ -453,9 +453,8 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op))
                      if args.storage is None else None,
-                     # achieved and traffic are both per step (at 7B: 3 launches of the block
-                     # kernel and one for the norm vectors): algorithmic bytes of a step /
-                     # device time of a step
+                     # achieved and traffic are both per step (at 7B: 2 launches of the block
+                     # kernel): algorithmic bytes of a step / device time of a step
                      "per": "step", "algorithmic_bytes": bpp * n_params,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},

@@ -63,7 +63,7 @@ struct TensorDesc {
 // The descriptors travel by value in the kernel arguments (112 bytes each; the runtime passes
 // arguments of this size intact).  Fewer, longer launches: each launch ends with a partly
 // filled round of workgroups, and small tensors would otherwise queue up behind each other.
-constexpr int kTensorsPerLaunch = 112;
+constexpr int kTensorsPerLaunch = 160;
 
 struct FusedParams {
     TensorDesc t[kTensorsPerLaunch];

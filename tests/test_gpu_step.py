@@ -69,8 +69,8 @@ CASES = [
     ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.05, 0.0, 0.0, 20480, 23),
     ([20480 * 2 + 4096, 20480], torch.bfloat16, 20, 64, 0.05, 0.0, 0.01, 20480, 22),
     ([20480 + 8192], torch.bfloat16, 24, 32, 0.05, 0.0, 0.0, 20480, 26),
-    # more tensors of one size class than one launch takes (112): two launches
-    ([96 + 8 * (i % 5) for i in range(130)] + [3000], torch.bfloat16, 3, 8, 0.05, 0.0, 0.0, 1024, 4),
+    # more tensors of one size class than one launch takes (160): two launches
+    ([96 + 8 * (i % 5) for i in range(190)] + [3000], torch.bfloat16, 3, 8, 0.05, 0.0, 0.0, 1024, 4),
 ]
 
 
