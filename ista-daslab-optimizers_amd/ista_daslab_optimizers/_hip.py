@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmicroadam_hip.so")
 
 MA_F32, MA_BF16 = 0, 1
+MA_ERR_ARG = -1
 MA_ERR_NOT_FUSABLE = -5
 MA_ERR_LDS = -6
 MA_ERR_WORKSPACE = -7

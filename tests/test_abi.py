@@ -75,6 +75,45 @@ def test_fused_step_check_rejects_bad_layouts():
     assert chk() == -3
 
 
+def test_step_checks_refuse_what_does_not_fit_in_lds():
+    """The admission checks lay out the LDS of the launch the tensor would get: a selection of
+    70 % of a 20480-element fp32 block needs more than the 160 KB a workgroup can have, so the
+    tensor is refused (and the optimizer then steps it op by op) instead of failing at launch."""
+    from ista_daslab_optimizers import _hip
+    import math
+    d = 20480 * 2
+    t = _hip.MaTensor()
+    for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
+        setattr(t, f, 0x10000)
+    t.d, t.lr, t.weight_decay, t.index = d, 1e-3, 0.0, 0
+    for k_init, want in ((0.01, 0), (0.7, _hip.MA_ERR_LDS)):
+        t.k = 2 * int(math.ceil(20480 * k_init))
+        h = _hip.MaHyper(1, 10, _hip.MA_F32, 64, 20480, k_init, 0.9, 0.999, 1e-8)
+        assert _hip.lib.ma_fused_step_check(ctypes.byref(t), ctypes.byref(h)) == want, k_init
+        h.quant_block_size = 40960
+        assert _hip.lib.ma_spanning_step_check(ctypes.byref(t), ctypes.byref(h), 0.5) == want, k_init
+
+
+def test_logged_step_argument_checks():
+    """Host-only: the size of the per-block buffer a logging step needs, and the refusals that
+    come before any launch."""
+    from ista_daslab_optimizers import _hip
+    t = _hip.MaTensor()
+    for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
+        setattr(t, f, 0x10000)
+    t.d, t.k, t.lr, t.weight_decay, t.index = 20480 * 2 + 4096, 205 * 2 + 41, 1e-3, 0.0, 0
+    h = _hip.MaHyper(1, 10, _hip.MA_BF16, 64, 20480, 0.01, 0.9, 0.999, 1e-8)
+    assert _hip.lib.ma_logged_step_partials(ctypes.byref(t), 1, ctypes.byref(h)) == 3 * 8
+    assert _hip.lib.ma_logged_step_partials(None, 1, ctypes.byref(h)) == -1
+    call = lambda route, partials, n, sums: _hip.lib.ma_logged_step(
+        route, ctypes.byref(t), 1, ctypes.byref(h), 0.0, None, 0, partials, n, sums, None)
+    assert call(_hip.MA_ROUTE_FUSED, 0x10000, 24, None) == _hip.MA_ERR_ARG        # no sums
+    assert call(_hip.MA_ROUTE_FUSED, 0x10000, 23, 0x10000) == _hip.MA_ERR_ARG     # buffer too short
+    assert call(_hip.MA_ROUTE_FUSED, None, 24, 0x10000) == _hip.MA_ERR_ARG
+    assert call(7, 0x10000, 24, 0x10000) == _hip.MA_ERR_ARG                       # unknown route
+    assert call(_hip.MA_ROUTE_DENSIFIED, 0x10000, 24, 0x10000) == _hip.MA_ERR_NOT_FUSABLE  # alpha 0
+
+
 def test_spanning_step_check_and_workspace():
     """Host-only validation of ma_spanning_step's conditions and its workspace size."""
     from ista_daslab_optimizers import _hip
