@@ -421,7 +421,8 @@ def main():
         ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    dev_ms = sorted(a.elapsed_time(b) for a, b in ev)
+    dev_series = [a.elapsed_time(b) for a, b in ev]  # in step order
+    dev_ms = sorted(dev_series)
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = sum(dev_ms) / len(dev_ms)
 
@@ -457,7 +458,8 @@ def main():
                      # kernel): algorithmic bytes of a step / device time of a step
                      "per": "step", "algorithmic_bytes": bpp * n_params,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
-                     "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2]},
+                     "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2],
+                     "device_ms_series": [round(x, 3) for x in dev_series]},
     }
     if not args.no_cpu_baseline:
         del grad_sets
