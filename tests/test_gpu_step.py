@@ -227,6 +227,57 @@ def test_lr_schedule_none_grads_and_closure(oracle):
             assert np.array_equal(to_np(p.data), oparams[i])
 
 
+def test_logging_with_mixed_types_and_missing_gradients(oracle):
+    """One list holding bf16 and fp32 tensors of all block classes, and on some logging steps a
+    tensor without a gradient: the step is then several library calls (one per route and element
+    type), whose kernels add their shares to the same six sums (micro_adam.py:121, 125-136,
+    328, 330)."""
+    from ista_daslab_optimizers import MicroAdam
+    gen = torch.Generator().manual_seed(21)
+    spec = [(20480 * 2 + 300, torch.bfloat16), (768, torch.bfloat16), (20480 + 8, torch.float32),
+            (3000, torch.float32), (10000, torch.bfloat16)]
+    cpu = [(torch.randn(n, generator=gen) * 0.02).to(dt) for n, dt in spec]
+    oparams = [to_np(p) for p in cpu]
+    oref = oracle.OracleMicroAdam(oparams, 4, 1e-3, 64, 0.01, 0, weight_decay=0.01)
+    gparams = [torch.nn.Parameter(p.clone().cuda()) for p in cpu]
+    opt = MicroAdam(gparams, m=4, lr=1e-3, quant_block_size=64, weight_decay=0.01)
+    opt.log_interval = 2
+    opt._logging_active = lambda: True
+    logged = []
+    opt._log = lambda *a: logged.append([float(x) for x in a[:6]])
+    calls = []
+    inner = opt._fused_step
+    opt._fused_step = lambda route, dtype, entries, sums=None: (
+        calls.append((opt.steps, dtype, len(entries), sums is not None)),
+        inner(route, dtype, entries, sums))
+    wanted = []
+    for s in range(6):
+        grads = [(torch.randn(n, generator=gen) * 1e-2).to(dt) for n, dt in spec]
+        if s in (1, 4):
+            grads[2] = None     # step 2 is a logging step, step 5 is not
+        for p, g in zip(gparams, grads):
+            p.grad = None if g is None else g.clone().cuda()
+        opt.step()
+        out = oref.step([None if g is None else to_np(g) for g in grads], metrics=(s + 1) % 2 == 0)
+        if out is not None:
+            wanted.append(out)
+        for i, p in enumerate(gparams):
+            if oref.state[i] is not None:
+                assert_state_equal(opt.state[p], oref.state[i], f"step {s + 1} tensor {i}")
+            assert np.array_equal(to_np(p.data), oparams[i]), f"step {s + 1} tensor {i}"
+    # two calls per step (bf16, fp32), with sums exactly on the logging steps
+    assert [c for c in calls if c[0] == 2] == [(2, torch.bfloat16, 3, True), (2, torch.float32, 1, True)]
+    assert [c for c in calls if c[0] == 3] == [(3, torch.bfloat16, 3, False), (3, torch.float32, 2, False)]
+    assert len(logged) == 3 == len(wanted)
+    keys = ("norm_qe", "norm_g", "norm_u", "norm_e", "sparsity_u", "sparsity_qe")
+    for got, want in zip(logged, wanted):
+        for key, value in zip(keys, got):
+            if key.startswith("sparsity"):
+                assert value == want[key], (key, value, want[key])
+            else:
+                assert value == pytest.approx(want[key], rel=1e-5, abs=0), (key, value, want[key])
+
+
 def test_state_layout_and_checkpoint_roundtrip():
     """State keys, dtypes and shapes as micro_adam.py:61-94; state_dict round trip, including
     the re-typing load_state_dict applies to floating-point state."""
