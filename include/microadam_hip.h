@@ -154,7 +154,7 @@ typedef struct ma_hyper {
  * top-k block: a = g + Qinv(e); block top-k -> I[index], V[index]; residual -> new min/max
  * and 4-bit codes; window -> Adam direction; p update (with decoupled weight decay).  The
  * caller advances st['index'] (MA:211) itself.  Conditions (else MA_ERR_NOT_FUSABLE, nothing
- * launched): quant_block_size a power of two in [8, 512] that divides d_block_size (or
+ * launched): quant_block_size a power of two in [8, 4096] that divides d_block_size (or
  * d <= d_block_size) and does not exceed d; p and g 16-byte aligned, error 4-byte aligned;
  * d_block_size a multiple of 8 unless d <= d_block_size. */
 int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
@@ -165,7 +165,7 @@ int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
 int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
 
 /* ma_fused_step for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), same
- * conditions, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and
+ * conditions but quant_block_size at most 512, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and
  * statistics; window -> Adam direction, + alpha * Qinv(e1); p update; the error feedback that is
  * stored is Q((1 - alpha) * Qinv(e1)) with statistics of its own. */
 int ma_fused_step_densified(const ma_tensor *tensors /* host */, int n_tensors,

@@ -621,6 +621,32 @@ struct FusedBlock {
         uint8_t *err = G.D.err + (G.e0 >> 1);
         uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
         uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+        // Quantisation blocks of 1024, 2048 or 4096 elements cover 2, 4 or 8 of the 512-element
+        // stretches a wave holds per chunk: every (wave, chunk) leaves its extremes in LDS
+        // (where the selection's histograms were), and each takes those of its block's stretches.
+        const bool long_q = QL == 0 && ql > kWave;
+        float *stretch = reinterpret_cast<float *>(hist);  // [wave * C + chunk][min, max]
+        if (long_q) {
+            __syncthreads();  // the selection may still be reading its lists there
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const int off = chunk_off<C>(wave, c, lane);
+                float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (FULL || off + e < n) {
+                        mn = fmin_raw(mn, r.val(c, e));
+                        mx = fmax_raw(mx, r.val(c, e));
+                    }
+                }
+                group_minmax<0>(mn, mx, kWave);
+                if (lane == 0) {
+                    stretch[(wave * C + c) * 2] = mn;
+                    stretch[(wave * C + c) * 2 + 1] = mx;
+                }
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -639,7 +665,18 @@ struct FusedBlock {
                     }
                 }
             }
-            group_minmax<QL>(mn, mx, ql);
+            if (long_q) {
+                const int per = ql / kWave;  // stretches per quantisation block
+                const int first = (wave * C + c) / per * per;
+                mn = INFINITY;
+                mx = -INFINITY;
+                for (int j = 0; j < per; ++j) {
+                    mn = fmin_raw(mn, stretch[(first + j) * 2]);
+                    mx = fmax_raw(mx, stretch[(first + j) * 2 + 1]);
+                }
+            } else {
+                group_minmax<QL>(mn, mx, ql);
+            }
             const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
             if (FULL || off < n) {
                 if ((lane & (ql - 1)) == 0) {

@@ -445,12 +445,13 @@ static int common_check(const ma_tensor *t, const ma_hyper *h, Geometry *g) {
     return 0;
 }
 
-static int fused_check(const ma_tensor *t, const ma_hyper *h) {
+// dense: with 0 < alpha < 1 (whose two quantisations stay inside a wave's stretch of 512)
+static int fused_check(const ma_tensor *t, const ma_hyper *h, bool dense = false) {
     Geometry g;
     const int rc = common_check(t, h, &g);
     if (rc) return rc;
     const int64_t q = h->quant_block_size;
-    if (q < 8 || q > 512 || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
+    if (q < 8 || q > (dense ? 512 : 4096) || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
     if (t->d < q) return MA_ERR_NOT_FUSABLE;
     const bool single = t->d <= h->d_block_size;
     if (!single && (g.dbs % q != 0 || g.dbs % 8 != 0)) return MA_ERR_NOT_FUSABLE;
@@ -730,7 +731,8 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     if ((aux & kAuxQuantErr) && (span || dense)) return MA_ERR_NOT_FUSABLE;
     if ((aux & kAuxLog) && !metrics) return MA_ERR_ARG;
     for (int i = 0; i < n_tensors; ++i) {
-        const int rc = span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h);
+        const int rc =
+            span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h, alpha > 0.0);
         if (rc) return rc;
     }
     if (n_tensors == 0) return 0;

@@ -221,7 +221,10 @@ class MicroAdam(torch.optim.Optimizer):
         if _hip.lib.ma_fused_step_check(ctypes.byref(probe), ctypes.byref(h)) == 0:
             if self.alpha == -2:
                 return FUSED_QUANT_ERR
-            return FUSED if self.alpha == 0 else FUSED_DENSIFIED
+            if self.alpha == 0:
+                return FUSED
+            if self.quant_block_size <= 512:  # (ma_fused_step_densified's own limit)
+                return FUSED_DENSIFIED
         if self.alpha == -2:
             return OP_BY_OP
         if _hip.lib.ma_spanning_step_check(ctypes.byref(probe), ctypes.byref(h),

@@ -69,6 +69,11 @@ CASES = [
     ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.05, 0.0, 0.0, 20480, 23),
     ([20480 * 2 + 4096, 20480], torch.bfloat16, 20, 64, 0.05, 0.0, 0.01, 20480, 22),
     ([20480 + 8192], torch.bfloat16, 24, 32, 0.05, 0.0, 0.0, 20480, 26),
+    # quantisation blocks longer than the 512 elements a wave holds per chunk
+    ([20480 * 2 + 4096, 3000, 12288], torch.bfloat16, 4, 1024, 0.01, 0.0, 0.0, 20480, 6),
+    ([20480 + 5000], torch.bfloat16, 10, 4096, 0.01, 0.0, 0.01, 20480, 12),
+    ([20480 + 2048 + 77, 4096], torch.float32, 3, 2048, 0.01, 0.0, 0.0, 20480, 5),
+    ([32768 + 9000], torch.bfloat16, 3, 4096, 0.01, 0.0, 0.0, 32768, 5),
     # more tensors of one size class than one launch takes (160): two launches
     ([96 + 8 * (i % 5) for i in range(190)] + [3000], torch.bfloat16, 3, 8, 0.05, 0.0, 0.0, 1024, 4),
 ]
@@ -87,6 +92,8 @@ GENERAL_CASES = [
     ([999], torch.float32, 2, 100, 0.03, 0.25, 0.01, 400, 5),
     ([20480 * 3 + 77], torch.bfloat16, 4, 100001, 0.01, 0.5, 0.0, 20480, 6),
     ([50, 20], torch.bfloat16, 3, 60, 0.1, 0.0, 0.0, 20480, 4),
+    # 0 < alpha < 1 with quantisation blocks between 512 elements and the top-k block
+    ([20480 * 2 + 4096], torch.bfloat16, 3, 1024, 0.01, 0.5, 0.0, 20480, 4),
     # alpha == -2 with quantisation blocks that the one-pass kernels do not take
     ([4100, 33], torch.bfloat16, 3, 1000, 0.01, -2, 0.0, 1024, 5),
 ]
@@ -105,6 +112,7 @@ QUANT_ERR_CASES = [
     ([20480 * 3, 1001], torch.bfloat16, 10, 64, 0.01, -2, 0.01, 20480, 12),
     ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.05, -2, 0.0, 20480, 22),
     ([20480 + 77], torch.float32, 5, 32, 0.01, -2, 0.0, 20480, 7),
+    ([20480 * 2 + 1000], torch.bfloat16, 4, 2048, 0.01, -2, 0.0, 20480, 6),
 ]
 
 
@@ -469,6 +477,7 @@ LOGGING_CASES = [
     ([20480 * 2 + 4096, 300], torch.bfloat16, 4, 64, -2, 0.01, "quant_err"),
     ([20480 + 77], torch.float32, 3, 32, -2, 0.0, "quant_err"),
     ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.0, 0.0, "fused"),   # 5 %: no coordinate cells
+    ([20480 * 2 + 3000], torch.bfloat16, 4, 2048, 0.0, 0.01, "fused"),  # long quantisation blocks
 ]
 
 
