@@ -2023,13 +2023,16 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             }
         } else if constexpr (PASS == 2) {
             fb.span_load_row(G);
-            fb.load_params_window(G);
+            fb.wide = fb.wide_window(G);
+            if (fb.wide) fb.load_window_wide(G); else fb.load_window(G);
+            fb.span_load_residual(G);
             fb.span_row_to_lds(G);
             fb.template span_statistics<true>(G, S);
             fb.window_cells(G);
-            // (asked for only now: held through the window stage, the residual would cost
-            // the registers that stage needs)
-            fb.span_load_residual(G);
+            // (asked for only now: the residual and the parameters both held through the
+            // window stage cost the registers that stage needs; the parameters are wanted
+            // last in the stage below, so they are the ones that wait)
+            fb.load_params(G);
             fb.span_param_stage(G, S);
         } else {
             fb.span_load_residual(G);
