@@ -1719,9 +1719,13 @@ struct FusedBlock {
             }
             const bool second = off >= S.bnd;
             const float mn = second ? mn1 : mn0, u = second ? u1 : u0;
+            // the nibbles as bytes of two words (even elements high), one conversion each, as
+            // in dequant
+            uint32_t odd = cw[c] & 0x0f0f0f0fu, even = (cw[c] >> 4) & 0x0f0f0f0fu;
+            asm volatile("" : "+v"(odd), "+v"(even));
 #pragma unroll
             for (int e = 0; e < kChunk; ++e) {
-                const uint32_t code = (cw[c] >> (8 * (e >> 1) + ((e & 1) ? 0 : 4))) & 15u;
+                const uint32_t code = (((e & 1) ? odd : even) >> (8 * (e >> 1))) & 0xffu;
                 float deq = (float)code * u;
                 deq = deq + mn;
                 v[e] = v[e] + deq;
