@@ -30,7 +30,7 @@ MEASURED_TRAFFIC = {
     ("llama2-7b", False): 50.729e9,     # profiles/fused_step_llama2-7b_hbm_traffic.txt
     ("gpt2-small", False): 0.938e9,     # profiles/fused_step_gpt2-small_hbm_traffic.txt
     ("outlier-1.3b", False): 15.276e9,  # profiles/fused_step_outlier-1.3b_hbm_traffic.txt
-    ("llama3-8b", False): 93.037e9,     # profiles/spanning_step_llama3-8b_hbm_traffic.txt
+    ("llama3-8b", False): 92.056e9,     # profiles/spanning_step_llama3-8b_hbm_traffic.txt
 }
 
 
