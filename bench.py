@@ -27,10 +27,10 @@ CAL_BYTES = 26214 * 40960  # --copy-calibration: bytes the known-size copy reads
 # counters read for a plain copy of known size; (workload, op_by_op) -> bytes.  The figures and
 # the commands behind them are in profiles/.
 MEASURED_TRAFFIC = {
-    ("llama2-7b", False): 50.729e9,     # profiles/fused_step_llama2-7b_hbm_traffic.txt
-    ("gpt2-small", False): 0.938e9,     # profiles/fused_step_gpt2-small_hbm_traffic.txt
-    ("outlier-1.3b", False): 15.276e9,  # profiles/fused_step_outlier-1.3b_hbm_traffic.txt
-    ("llama3-8b", False): 92.056e9,     # profiles/spanning_step_llama3-8b_hbm_traffic.txt
+    ("llama2-7b", False): (50.729e9, "profiles/fused_step_llama2-7b_hbm_traffic.txt"),
+    ("gpt2-small", False): (0.938e9, "profiles/fused_step_gpt2-small_hbm_traffic.txt"),
+    ("outlier-1.3b", False): (15.276e9, "profiles/fused_step_outlier-1.3b_hbm_traffic.txt"),
+    ("llama3-8b", False): (92.056e9, "profiles/spanning_step_llama3-8b_hbm_traffic.txt"),
 }
 
 
@@ -79,6 +79,31 @@ WORKLOADS = {
     # not one of the five either: the 7B list with alpha > 0 and short quantisation blocks
     "llama2-7b-alpha": (llama2_7b, "bf16", 10, 0.01, 64, 0.5, 1e-3),
 }
+
+
+_probe = None
+
+
+def stream_probe():
+    """ma_stream_probe of libmicroadam_probe.so (csrc/stream_probe.h): known-size streaming
+    kernels, measurement tooling that only this benchmark loads."""
+    global _probe
+    if _probe is None:
+        import ctypes
+        path = os.path.join(ROOT, "ista-daslab-optimizers_amd", "ista_daslab_optimizers",
+                            "libmicroadam_probe.so")
+        fn = ctypes.CDLL(path).ma_stream_probe
+        vp = ctypes.c_void_p
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, vp, vp, vp, vp,
+                       vp, vp]
+
+        def call(*args):
+            rc = fn(*args)
+            if rc:
+                raise RuntimeError(f"ma_stream_probe failed with code {rc}")
+        _probe = call
+    return _probe
 
 
 def numel(shape):
@@ -289,9 +314,8 @@ def calibration(args):
 
     def probe(mode, nt, wgs=0):
         def run():
-            _hip.check(_hip.lib.ma_stream_probe(mode, nt, nbytes, wgs, a.data_ptr(), b.data_ptr(),
-                                                c.data_ptr(), e.data_ptr(), sink.data_ptr(),
-                                                _hip.stream_ptr()), "ma_stream_probe")
+            stream_probe()(mode, nt, nbytes, wgs, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                           e.data_ptr(), sink.data_ptr(), _hip.stream_ptr())
         return run
 
     moved = {0: nbytes, 1: nbytes, 2: 2 * nbytes, 3: 3 * nbytes, 4: 3 * nbytes + nbytes // 2}
@@ -343,6 +367,11 @@ def main():
     ap.add_argument("--calibration", action="store_true",
                     help="time known-size streaming kernels instead of the optimizer step")
     ap.add_argument("--calibration-gib", type=int, default=4, help="bytes per array, GiB")
+    ap.add_argument("--grad-scale-drift", type=float, default=0.0,
+                    help="multiply the gradients of step i by (1 + drift)^i (set on the device "
+                         "before the step, outside the timed kernels): with a drift well above the "
+                         "1/32 margin of the hinted top-k selection its bound fails in every block "
+                         "and the step pays the fallback selection")
     ap.add_argument("--storage", choices=["bf16", "f32"], default=None,
                     help="override the element type of parameters and gradients")
     args = ap.parse_args()
@@ -389,6 +418,16 @@ def main():
                     betas=(0.9, 0.999), eps=1e-8, weight_decay=0)
     opt.use_fused = not args.op_by_op
 
+    scale_of = {}
+
+    def prepare(i):
+        """--grad-scale-drift: the gradient set of step i brought to that step's level."""
+        if args.grad_scale_drift:
+            which = i % len(grad_sets)
+            now = (1.0 + args.grad_scale_drift) ** i
+            torch._foreach_mul_(grad_sets[which], now / scale_of.get(which, 1.0))
+            scale_of[which] = now
+
     def one_step(i):
         gs = grad_sets[i % len(grad_sets)]
         for p, g in zip(params, gs):
@@ -396,6 +435,7 @@ def main():
         opt.step()
 
     for i in range(args.warmup):
+        prepare(i)
         one_step(i)
     torch.cuda.synchronize()
     if args.copy_calibration:
@@ -404,9 +444,8 @@ def main():
         src = torch.empty(CAL_BYTES // 2, dtype=torch.bfloat16, device=dev).normal_()
         dst = torch.empty_like(src)
         sink = torch.zeros(1, dtype=torch.int32, device=dev)
-        _hip.check(_hip.lib.ma_stream_probe(2, 1, CAL_BYTES, 0, src.data_ptr(), None, dst.data_ptr(),
-                                            None, sink.data_ptr(), _hip.stream_ptr()),
-                   "ma_stream_probe")
+        stream_probe()(2, 1, CAL_BYTES, 0, src.data_ptr(), None, dst.data_ptr(), None,
+                       sink.data_ptr(), _hip.stream_ptr())
         torch.cuda.synchronize()
         del src, dst
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
@@ -414,6 +453,7 @@ def main():
     host = 0.0  # time the host spends inside step() (the kernels run behind it)
     t0 = time.perf_counter()
     for i in range(args.steps):
+        prepare(args.warmup + i)  # (its kernels run between the events of two steps)
         ev[i][0].record()
         h0 = time.perf_counter()
         one_step(args.warmup + i)
@@ -426,6 +466,9 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = sum(dev_ms) / len(dev_ms)
 
+    traffic, traffic_source = (MEASURED_TRAFFIC.get((args.workload, args.op_by_op), (None, None))
+                               if args.storage is None and not args.grad_scale_drift
+                               else (None, None))
     bpp = algorithmic_bytes_per_param(shapes, dtype, m, k_init, q, alpha, opt.d_block_size,
                                       args.warmup + 1, args.steps)
     achieved = bpp * n_params / (kernel_ms * 1e-3) / 1e9
@@ -448,12 +491,13 @@ def main():
                    "grad_sets": args.grad_sets,
                    "tensors": len(shapes), "m": m,
                    "k_init": k_init, "quant_block_size": q, "alpha": alpha,
-                   "d_block_size": opt.d_block_size,
+                   "d_block_size": opt.d_block_size, "grad_scale_drift": args.grad_scale_drift,
                    "route": route_label(opt, params)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.op_by_op))
-                     if args.storage is None else None,
+                     # counters cannot be read from inside this run: the figure is the one the
+                     # same workload measured under rocprofv3 --pmc, kept in the file named
+                     "traffic": traffic, "traffic_source": traffic_source,
                      # achieved and traffic are both per step (at 7B: 2 launches of the block
                      # kernel): algorithmic bytes of a step / device time of a step
                      "per": "step", "algorithmic_bytes": bpp * n_params,

@@ -138,6 +138,9 @@ typedef struct ma_tensor {
     double weight_decay; /* group['weight_decay'],                     MA:122 */
     int32_t index;      /* st['index'], the ring row written by this step, MA:180 */
     int32_t reserved;
+    void *quant_err;    /* st['quant_err'], `dtype`, d elements, MA:67-68; written by
+                           ma_fused_step_quant_err (and ma_logged_step on that route), 16-byte
+                           aligned; the other entry points ignore it (may be NULL) */
 } ma_tensor;
 
 typedef struct ma_hyper {
@@ -219,8 +222,10 @@ int ma_spanning_step_static(const ma_tensor *tensors /* host */, int n_tensors,
 /* ma_fused_step for alpha == -2 (densify_update_using_quant_error, MA:238-273), same conditions,
  * still one pass per top-k block: with the residual a and the new error feedback e in
  * registers, p = p * (1 - lr * wd) (MA:234-235), p = p - a (MA:264), p = p + Qinv(e) (MA:269),
- * each rounded to the parameter's type, then the Adam step as for alpha == 0.  st['quant_err']
- * (MA:258-270, read by the logged norms only) is not written. */
+ * each rounded to the parameter's type, then the Adam step as for alpha == 0.  Every step
+ * rewrites st['quant_err'] = a - Qinv(e), rounded to the parameter's type (MA:258-271); a tensor
+ * whose quant_err pointer is NULL or not 16-byte aligned is rejected (MA_ERR_ARG /
+ * MA_ERR_NOT_FUSABLE) before anything is launched. */
 int ma_fused_step_quant_err(const ma_tensor *tensors /* host */, int n_tensors,
                             const ma_hyper *hyper /* host */, void *stream);
 
@@ -290,22 +295,6 @@ int ma_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d
 int ma_copy_values_typed(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
                          const int16_t *indices, const void *inp, void *out, int direction,
                          int dtype, int values_dtype, void *stream);
-
-/* ---- calibration of measurements ------------------------------------------------------------- */
-
-/* No counterpart in the reference.  Streams `bytes` (a multiple of 40960) of each array it
- * touches with the fused step's own access shape: 512-thread workgroups that each own one
- * contiguous 40 KiB stretch and move it as 16-byte accesses, a contiguous KiB per wave.
- * mode 0: reads a.  1: writes c.  2: c = a.  3: b = a + b (two reads, one write).
- * 4: reads a, b and e, writes b and e, with e a quarter as long as a (the step's gradient,
- *    parameter and 4-bit error-feedback streams: 7 bytes per bf16 element).
- * nontemporal != 0 uses the cache-bypassing loads and stores the step uses.  workgroups > 0
- * caps the grid (each workgroup then takes several stretches in turn), 0 launches one per
- * stretch.  sink: 4 bytes of device memory (keeps the read-only mode's loads alive).  Used by
- * bench.py --calibration: the HBM counters are scaled by what they read for these kernels, and
- * the rates they reach are this device's ceiling for the step's traffic. */
-int ma_stream_probe(int mode, int nontemporal, int64_t bytes, int64_t workgroups, const void *a,
-                    void *b, void *c, void *e, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

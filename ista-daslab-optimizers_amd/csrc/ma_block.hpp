@@ -58,7 +58,8 @@ struct TensorDesc {
     float decay;
     int32_t apply_decay;
     int32_t blk0;         // block of the tensor that its first work item stands for
-    float *ws;            // two-pass route: per-block extremes of the residual, else unused
+    float *ws;            // two-pass route: per-block extremes of the residual;
+                          // alpha == -2: st['quant_err'] (elements of the data's type); else unused
 };
 // The descriptors travel by value in the kernel arguments (112 bytes each; the runtime passes
 // arguments of this size intact).  Fewer, longer launches: each launch ends with a partly
@@ -712,7 +713,7 @@ struct FusedBlock {
     __device__ __forceinline__ void quant_err_chunk(const BlockGeo &G, int c, int off, int n,
                                                     const float (&x)[8], const float (&cf)[8],
                                                     float mnf, float u) {
-        float pv[8];
+        float pv[8], lost[8];
         if constexpr (QE) praw[c].to_float(pv);
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
@@ -721,18 +722,24 @@ struct FusedBlock {
             const float d = to_elem(0.0f + deq);
             const bool valid = FULL || off + e < n;
             if (valid) log_square(kMtError, d);
+            lost[e] = 0.0f;
             if constexpr (QE) {
                 if (G.D.apply_decay != 0) pv[e] = to_elem(pv[e] * G.D.decay);
                 pv[e] = to_elem(pv[e] + (-1.0f) * x[e]);
                 pv[e] = to_elem(pv[e] + d);
                 if (valid) {
-                    const float lost = to_elem(x[e] - d);
-                    log_square(kMtQuantErr, lost);
-                    log_zero(kMtQuantErrZeros, lost);
+                    lost[e] = to_elem(x[e] - d);
+                    log_square(kMtQuantErr, lost[e]);
+                    log_zero(kMtQuantErrZeros, lost[e]);
                 }
             }
         }
-        if constexpr (QE) praw[c].from_float(pv);
+        if constexpr (QE) {
+            praw[c].from_float(pv);
+            // st['quant_err'] = a - Qinv(e) (MA:259-271)
+            store8(reinterpret_cast<elem_t *>(G.D.ws) + G.e0, off, FULL ? 0x7fffffff : n, true,
+                   lost);
+        }
     }
 
     // the weight decay of the update stages: with alpha == -2 it has been applied already
@@ -2065,8 +2072,6 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
 
 constexpr int kLdsLimit = 160 * 1024;
 
-static inline int launch_status() { return (int)hipGetLastError(); }
-
 
 template <class K>
 static int allow_big_lds(K kernel, int bytes) {
@@ -2085,10 +2090,11 @@ static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const F
     // kernels with extras, take the budget of two
     constexpr int kWaves_ =
         (R::kBF16 && R::kC <= kClass2 && !HOLD && AUX == 0) ? kWavesThreeWG : kMinWaves;
-    int rc = allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, lds_bytes);
-    if (rc) return rc;
-    fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX><<<grid, kWG, lds_bytes, s>>>(P);
-    return launch_status();
+    // grid == 0: the preparation of the launch only (whatever may fail apart from the launch
+    // itself), so that a call can prepare all its launches before the first one starts
+    if (grid == 0) return allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, lds_bytes);
+    return launch_kernel(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, dim3(grid), kWG,
+                         lds_bytes, s, P);
 }
 
 // the kernels with extras (logging, alpha == -2): one per class, any quantisation group
@@ -2148,28 +2154,21 @@ static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s
     // the first pass has the register needs of the fused kernel
     constexpr int kFirst =
         (R::kBF16 && R::kC <= kClass2 && AUX == 0) ? kWavesThreeWG : kMinWaves;
-    int rc;
+    // grid == 0: the preparation only, as in launch_fused_one
     switch (pass) {
         case 1:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 1, AUX>, lds_bytes);
-            if (rc) return rc;
-            span_step_kernel<R, kFirst, 1, AUX><<<grid, kWG, lds_bytes, s>>>(P);
-            break;
+            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 1, AUX>, lds_bytes);
+            return launch_kernel(span_step_kernel<R, kFirst, 1, AUX>, dim3(grid), kWG, lds_bytes, s, P);
         case 2:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 2, AUX>, lds_bytes);
-            if (rc) return rc;
-            span_step_kernel<R, kFirst, 2, AUX><<<grid, kWG, lds_bytes, s>>>(P);
-            break;
+            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 2, AUX>, lds_bytes);
+            return launch_kernel(span_step_kernel<R, kFirst, 2, AUX>, dim3(grid), kWG, lds_bytes, s, P);
         case 4:
-            rc = allow_big_lds(span_step_kernel<R, kFirst, 4, AUX>, lds_bytes);
-            if (rc) return rc;
-            span_step_kernel<R, kFirst, 4, AUX><<<grid, kWG, lds_bytes, s>>>(P);
-            break;
+            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 4, AUX>, lds_bytes);
+            return launch_kernel(span_step_kernel<R, kFirst, 4, AUX>, dim3(grid), kWG, lds_bytes, s, P);
         default:  // needs the kSh* words only
-            span_step_kernel<R, kMinWaves, 3, AUX><<<grid, kWG, kMiscBytes, s>>>(P);
-            break;
+            if (grid == 0) return 0;
+            return launch_kernel(span_step_kernel<R, kMinWaves, 3, AUX>, dim3(grid), kWG, kMiscBytes, s, P);
     }
-    return launch_status();
 }
 
 template <template <int> class RT, int AUX = 0>

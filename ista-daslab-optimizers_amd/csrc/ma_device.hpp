@@ -12,6 +12,22 @@
 
 namespace ma {
 
+// Launches `kernel` and returns what the runtime says about THIS launch (0, or a hipError_t).
+// The arguments are converted to the kernel's own parameter types.  (The <<< >>> form reports
+// nothing itself, and hipGetLastError() after it returns, and clears, whatever error any earlier
+// call of the thread left behind.)
+template <class T>
+struct launch_arg {
+    typedef T type;
+};
+template <class... P>
+static inline int launch_kernel(void (*kernel)(P...), dim3 grid, unsigned block, size_t lds_bytes,
+                                hipStream_t stream, typename launch_arg<P>::type... args) {
+    void *argv[] = {const_cast<void *>(static_cast<const void *>(&args))...};
+    return (int)hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, dim3(block), argv,
+                                lds_bytes, stream);
+}
+
 constexpr int kWG = 512;  // threads per workgroup of the block kernels
 constexpr int kWave = 64;
 constexpr int kWaves = kWG / kWave;

@@ -396,10 +396,9 @@ static int launch_topk(int C, unsigned grid, int lds_bytes, hipStream_t s, int64
     case CC: {                                                                               \
         int rc = allow_big_lds(block_topk_kernel<RT<CC>>, lds_bytes);                        \
         if (rc) return rc;                                                                   \
-        block_topk_kernel<RT<CC>><<<grid, kWG, lds_bytes, s>>>(                              \
-            d, dbs, k_many, k_few, (typename RT<CC>::elem_t *)x, I_row, V_row, zero_selected, \
-            L);                                                                              \
-        return launch_status();                                                              \
+        return launch_kernel(block_topk_kernel<RT<CC>>, dim3(grid), kWG, lds_bytes, s, d,    \
+                             dbs, k_many, k_few, (typename RT<CC>::elem_t *)x, I_row, V_row, \
+                             zero_selected, L);                                              \
     }
     switch (C) {
         MA_TOPK_CASE(kClass0)
@@ -524,9 +523,9 @@ int ma_get_max_floats_for_shared_memory_per_thread_block(void) {
 }
 
 #define MA_DISPATCH_DTYPE(dtype, CALL_F32, CALL_BF16) \
-    if ((dtype) == MA_F32) { CALL_F32; }              \
-    else if ((dtype) == MA_BF16) { CALL_BF16; }       \
-    else return MA_ERR_ARG;
+    if ((dtype) == MA_F32) return CALL_F32;           \
+    if ((dtype) == MA_BF16) return CALL_BF16;         \
+    return MA_ERR_ARG;
 
 int ma_copy_values(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
                    const int16_t *indices, const void *inp, void *out, int direction, int dtype,
@@ -541,11 +540,10 @@ int ma_copy_values(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_s
     if (k == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     MA_DISPATCH_DTYPE(dtype,
-        (copy_values_kernel<float><<<grid_for(k), kWG, 0, s>>>(k, d_block_size, k_block_size,
-                                                                indices, inp, out, direction)),
-        (copy_values_kernel<uint16_t><<<grid_for(k), kWG, 0, s>>>(k, d_block_size, k_block_size,
-                                                                   indices, inp, out, direction)))
-    return launch_status();
+        launch_kernel(copy_values_kernel<float>, dim3(grid_for(k)), kWG, 0, s, k, d_block_size,
+                      k_block_size, indices, inp, out, direction),
+        launch_kernel(copy_values_kernel<uint16_t>, dim3(grid_for(k)), kWG, 0, s, k, d_block_size,
+                      k_block_size, indices, inp, out, direction))
 }
 
 int ma_zerorize_block_components(void *vector, const int16_t *indices, int64_t d, int64_t k,
@@ -559,11 +557,10 @@ int ma_zerorize_block_components(void *vector, const int16_t *indices, int64_t d
     if (k == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     MA_DISPATCH_DTYPE(dtype,
-        (zerorize_kernel<float><<<grid_for(k), kWG, 0, s>>>((float *)vector, indices, k,
-                                                            d_block_size, k_block_size)),
-        (zerorize_kernel<uint16_t><<<grid_for(k), kWG, 0, s>>>((uint16_t *)vector, indices, k,
-                                                               d_block_size, k_block_size)))
-    return launch_status();
+        launch_kernel(zerorize_kernel<float>, dim3(grid_for(k)), kWG, 0, s, (float *)vector,
+                      indices, k, d_block_size, k_block_size),
+        launch_kernel(zerorize_kernel<uint16_t>, dim3(grid_for(k)), kWG, 0, s, (uint16_t *)vector,
+                      indices, k, d_block_size, k_block_size))
 }
 
 int ma_asymm_block_quant(int64_t d, int64_t q, uint8_t *xq, const uint16_t *xmin,
@@ -572,9 +569,10 @@ int ma_asymm_block_quant(int64_t d, int64_t q, uint8_t *xq, const uint16_t *xmin
     hipStream_t s = (hipStream_t)stream;
     const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
     MA_DISPATCH_DTYPE(dtype,
-        (quant_kernel<float><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (const float *)x)),
-        (quant_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (const uint16_t *)x)))
-    return launch_status();
+        launch_kernel(quant_kernel<float>, dim3(grid), kWG, 0, s, d, q, xq, xmin, xmax,
+                      (const float *)x),
+        launch_kernel(quant_kernel<uint16_t>, dim3(grid), kWG, 0, s, d, q, xq, xmin, xmax,
+                      (const uint16_t *)x))
 }
 
 int ma_asymm_block_quant_inv(int64_t d, int64_t q, const uint8_t *xq, const uint16_t *xmin,
@@ -584,10 +582,10 @@ int ma_asymm_block_quant_inv(int64_t d, int64_t q, const uint8_t *xq, const uint
     hipStream_t s = (hipStream_t)stream;
     const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
     MA_DISPATCH_DTYPE(dtype,
-        (quant_inv_kernel<float><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (float *)x, alpha)),
-        (quant_inv_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, xq, xmin, xmax, (uint16_t *)x,
-                                                         alpha)))
-    return launch_status();
+        launch_kernel(quant_inv_kernel<float>, dim3(grid), kWG, 0, s, d, q, xq, xmin, xmax,
+                      (float *)x, alpha),
+        launch_kernel(quant_inv_kernel<uint16_t>, dim3(grid), kWG, 0, s, d, q, xq, xmin, xmax,
+                      (uint16_t *)x, alpha))
 }
 
 int ma_block_minmax(int64_t d, int64_t q, const void *x, uint16_t *xmin, uint16_t *xmax,
@@ -600,11 +598,10 @@ int ma_block_minmax(int64_t d, int64_t q, const void *x, uint16_t *xmin, uint16_
     if (wgs > 65536 * 16) wgs = 65536 * 16;
     const unsigned grid = (unsigned)wgs;
     MA_DISPATCH_DTYPE(dtype,
-        (minmax_kernel<float><<<grid, kWG, 0, s>>>(d, q, nblocks, (const float *)x, xmin, xmax,
-                                                   per_wave)),
-        (minmax_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, q, nblocks, (const uint16_t *)x, xmin,
-                                                      xmax, per_wave)))
-    return launch_status();
+        launch_kernel(minmax_kernel<float>, dim3(grid), kWG, 0, s, d, q, nblocks,
+                      (const float *)x, xmin, xmax, per_wave),
+        launch_kernel(minmax_kernel<uint16_t>, dim3(grid), kWG, 0, s, d, q, nblocks,
+                      (const uint16_t *)x, xmin, xmax, per_wave))
 }
 
 int ma_param_update(int64_t d, void *p, const void *u, float neg_lr, int apply_decay, float decay,
@@ -613,12 +610,10 @@ int ma_param_update(int64_t d, void *p, const void *u, float neg_lr, int apply_d
     hipStream_t s = (hipStream_t)stream;
     const unsigned grid = grid_for((d + kChunk - 1) / kChunk);
     MA_DISPATCH_DTYPE(dtype,
-        (param_update_kernel<float><<<grid, kWG, 0, s>>>(d, (float *)p, (const float *)u, neg_lr,
-                                                         apply_decay, decay)),
-        (param_update_kernel<uint16_t><<<grid, kWG, 0, s>>>(d, (uint16_t *)p,
-                                                            (const uint16_t *)u, neg_lr,
-                                                            apply_decay, decay)))
-    return launch_status();
+        launch_kernel(param_update_kernel<float>, dim3(grid), kWG, 0, s, d, (float *)p,
+                      (const float *)u, neg_lr, apply_decay, decay),
+        launch_kernel(param_update_kernel<uint16_t>, dim3(grid), kWG, 0, s, d, (uint16_t *)p,
+                      (const uint16_t *)u, neg_lr, apply_decay, decay))
 }
 
 int ma_block_topk(int64_t d, int64_t d_block_size, int64_t k_many, int64_t k_few, void *x,
@@ -664,14 +659,14 @@ int ma_compute_microadam_update(int blocks, int threads, int carveout, int64_t t
     int rc;
     if (dtype == MA_F32) {
         if ((rc = allow_big_lds(window_update_kernel<float>, L.total))) return rc;
-        window_update_kernel<float><<<(unsigned)nblocks, kWG, L.total, s>>>(
-            d, (int)d_block_size, (int)k_block_size, k, indices, values, (float *)out, W, L);
-    } else {
-        if ((rc = allow_big_lds(window_update_kernel<uint16_t>, L.total))) return rc;
-        window_update_kernel<uint16_t><<<(unsigned)nblocks, kWG, L.total, s>>>(
-            d, (int)d_block_size, (int)k_block_size, k, indices, values, (uint16_t *)out, W, L);
+        return launch_kernel(window_update_kernel<float>, dim3((unsigned)nblocks), kWG, L.total, s,
+                             d, (int)d_block_size, (int)k_block_size, k, indices, values,
+                             (float *)out, W, L);
     }
-    return launch_status();
+    if ((rc = allow_big_lds(window_update_kernel<uint16_t>, L.total))) return rc;
+    return launch_kernel(window_update_kernel<uint16_t>, dim3((unsigned)nblocks), kWG, L.total, s,
+                         d, (int)d_block_size, (int)k_block_size, k, indices, values,
+                         (uint16_t *)out, W, L);
 }
 
 int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
@@ -734,6 +729,10 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
         const int rc =
             span ? span_check(&tensors[i], h, alpha) : fused_check(&tensors[i], h, alpha > 0.0);
         if (rc) return rc;
+        if (aux & kAuxQuantErr) {  // st['quant_err'] is written with 16-byte stores
+            if (!tensors[i].quant_err) return MA_ERR_ARG;
+            if (((uintptr_t)tensors[i].quant_err & 15) != 0) return MA_ERR_NOT_FUSABLE;
+        }
     }
     if (n_tensors == 0) return 0;
     if (span) {
@@ -835,7 +834,8 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             D.apply_decay = t.weight_decay > 0.0 ? 1 : 0;
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
             D.blk0 = 0;
-            D.ws = span ? reinterpret_cast<float *>(static_cast<char *>(ws) + ws_here) : nullptr;
+            D.ws = span ? reinterpret_cast<float *>(static_cast<char *>(ws) + ws_here)
+                        : (aux & kAuxQuantErr) ? static_cast<float *>(t.quant_err) : nullptr;
             items += nb;
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
@@ -845,9 +845,12 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
         if (rc) return rc;
     }
 
+    // Two rounds over the plan: the first prepares every launch (kernel attributes: all that
+    // can fail apart from a launch itself), the second launches.
+    for (int round = 0; round < 2; ++round)
     for (const PlannedLaunch &L : plan) {
         const FusedParams &P = L.P;
-        const unsigned grid = (unsigned)P.total_items;
+        const unsigned grid = round == 0 ? 0u : (unsigned)P.total_items;
         const bool bf16 = h->dtype == MA_BF16;
         int rc = 0;
         if (dense && aux) {
@@ -873,7 +876,9 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                               : launch_span_f32(L.C, passes[i], grid, P.L.total, s, P);
             }
         }
-        if (rc) return rc;  // the runtime refused a launch: earlier launches of the call stand
+        // A launch the runtime refuses after an earlier one of the same call has started leaves
+        // the step applied to some tensors only: such an error is not one to retry after.
+        if (rc) return rc;
     }
     return 0;
 }
@@ -930,8 +935,8 @@ int ma_logged_step(int route, const ma_tensor *tensors, int n_tensors, const ma_
             return MA_ERR_ARG;
     }
     if (rc || blocks == 0) return rc;
-    metrics_reduce_kernel<<<1, kReduceThreads, 0, (hipStream_t)stream>>>(partials, blocks, sums);
-    return (int)hipGetLastError();
+    return launch_kernel(metrics_reduce_kernel, dim3(1), kReduceThreads, 0, (hipStream_t)stream,
+                         partials, blocks, sums);
 }
 
 int ma_spanning_step_check(const ma_tensor *tensor, const ma_hyper *hyper, double alpha) {

@@ -286,15 +286,15 @@ int ma_sparse_scalar_products(int64_t d, int64_t m_rows, int64_t k, int64_t d_bl
     gy = gy < 1 ? 1 : gy;
 #define CALL(TG, TV)                                                                            \
     if ((rc = allow_lds(sparse_dot_kernel<TG, TV>, lds))) return rc;                            \
-    sparse_dot_kernel<TG, TV><<<dim3((unsigned)nblocks, gy), kWG, lds, s>>>(                         \
-        d, (int)d_block_size, (int)k_block_size, k, (int)m_rows, (const TG *)g, indices,        \
-        (const TV *)values, partial);
+    rc = launch_kernel(sparse_dot_kernel<TG, TV>, dim3((unsigned)nblocks, (unsigned)gy), kWG,   \
+                       lds, s, d, (int)d_block_size, (int)k_block_size, k, (int)m_rows,         \
+                       (const TG *)g, indices, (const TV *)values, partial);
     MA_DISPATCH2(g_dtype, values_dtype, CALL)
 #undef CALL
-    if ((rc = (int)hipGetLastError())) return rc;
+    if (rc) return rc;
     const unsigned rgrid = (unsigned)((m_rows + kWG / 64 - 1) / (kWG / 64));
-    sparse_dot_reduce_kernel<<<rgrid, kWG, 0, s>>>(partial, nblocks, (int)m_rows, out);
-    return (int)hipGetLastError();
+    return launch_kernel(sparse_dot_reduce_kernel, dim3(rgrid), kWG, 0, s, partial, nblocks,
+                         (int)m_rows, out);
 }
 
 int ma_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d_block_size,
@@ -314,15 +314,15 @@ int ma_sparse_linear_combination(int64_t d, int64_t m_rows, int64_t k, int64_t d
     // waves instead of eight
 #define CALL_WG(TO, TV, WG)                                                                     \
     if ((rc = allow_lds(sparse_combine_kernel<TO, TV, WG>, lds))) return rc;                    \
-    sparse_combine_kernel<TO, TV, WG><<<(unsigned)nblocks, WG, lds, s>>>(                       \
-        d, (int)d_block_size, (int)k_block_size, k, (int)m_rows, coef, indices,                 \
-        (const TV *)values, (TO *)out);
+    rc = launch_kernel(sparse_combine_kernel<TO, TV, WG>, dim3((unsigned)nblocks), WG, lds, s,  \
+                       d, (int)d_block_size, (int)k_block_size, k, (int)m_rows, coef, indices,  \
+                       (const TV *)values, (TO *)out);
 #define CALL(TO, TV)                                                                            \
     if (k_block_size <= 256) { CALL_WG(TO, TV, 256) } else { CALL_WG(TO, TV, kWG) }
     MA_DISPATCH2(out_dtype, values_dtype, CALL)
 #undef CALL
 #undef CALL_WG
-    return (int)hipGetLastError();
+    return rc;
 }
 
 int ma_copy_values_typed(int64_t d, int64_t k, int64_t d_block_size, int64_t k_block_size,
@@ -339,11 +339,12 @@ int ma_copy_values_typed(int64_t d, int64_t k, int64_t d_block_size, int64_t k_b
     hipStream_t s = (hipStream_t)stream;
     const unsigned grid = (unsigned)((k + kWG - 1) / kWG);
 #define CALL(TD, TV)                                                                   \
-    copy_values_typed_kernel<TD, TV><<<grid, kWG, 0, s>>>(k, d_block_size, k_block_size, \
-                                                          indices, inp, out, direction);
+    rc = launch_kernel(copy_values_typed_kernel<TD, TV>, dim3(grid), kWG, 0, s, k,     \
+                       d_block_size, k_block_size, indices, inp, out, direction);
+    int rc = 0;
     MA_DISPATCH2(dtype, values_dtype, CALL)
 #undef CALL
-    return (int)hipGetLastError();
+    return rc;
 }
 
 }  // extern "C"

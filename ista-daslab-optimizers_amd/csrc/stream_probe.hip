@@ -1,16 +1,18 @@
 // Streaming kernels of known size, used to calibrate measurements of the MicroAdam step: what
 // the HBM counters read per byte, and what rate this device sustains for the step's own access
 // shape (512-thread workgroups, each owning one contiguous 40 KiB stretch of every array and
-// moving it as five 16-byte accesses per lane, a contiguous KiB per wave and access).  Part of
-// libmicroadam_hip.so; no counterpart in the reference.
+// moving it as five 16-byte accesses per lane, a contiguous KiB per wave and access).  Built
+// into a library of its own, libmicroadam_probe.so, which only the benchmark loads; no
+// counterpart in the reference.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../include/microadam_hip.h"
+#include "stream_probe.h"
 
 namespace ma {
 namespace {
 
+constexpr int kProbeErrArg = -1;  // bad argument
 constexpr int kThreads = 512;
 constexpr int kChunks = 5;
 constexpr int kSegBytes = kThreads * kChunks * 16;  // 40 KiB per workgroup and array
@@ -64,15 +66,13 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(const u4 *a, u4 *b, u4
 template <int MODE>
 int launch(bool nt, unsigned grid, hipStream_t s, const void *a, void *b, void *c, void *e,
            int64_t segments, void *sink) {
-    if (nt)
-        stream_kernel<MODE, true><<<grid, kThreads, 0, s>>>((const u4 *)a, (u4 *)b, (u4 *)c,
-                                                             (uint32_t *)e, segments,
-                                                             (uint32_t *)sink);
-    else
-        stream_kernel<MODE, false><<<grid, kThreads, 0, s>>>((const u4 *)a, (u4 *)b, (u4 *)c,
-                                                              (uint32_t *)e, segments,
-                                                              (uint32_t *)sink);
-    return (int)hipGetLastError();
+    const u4 *pa = (const u4 *)a;
+    u4 *pb = (u4 *)b, *pc = (u4 *)c;
+    uint32_t *pe = (uint32_t *)e, *ps = (uint32_t *)sink;
+    void *argv[] = {&pa, &pb, &pc, &pe, &segments, &ps};
+    const void *kernel = nt ? reinterpret_cast<const void *>(stream_kernel<MODE, true>)
+                            : reinterpret_cast<const void *>(stream_kernel<MODE, false>);
+    return (int)hipLaunchKernel(kernel, dim3(grid), dim3(kThreads), argv, 0, s);
 }
 
 }  // namespace
@@ -82,12 +82,12 @@ extern "C" int ma_stream_probe(int mode, int nontemporal, int64_t bytes, int64_t
                                const void *a, void *b, void *c, void *e, void *sink,
                                void *stream) {
     using namespace ma;
-    if (bytes <= 0 || bytes % kSegBytes != 0 || !sink) return MA_ERR_ARG;
+    if (bytes <= 0 || bytes % kSegBytes != 0 || !sink) return kProbeErrArg;
     const int64_t segments = bytes / kSegBytes;
-    if (segments > 0x7fffffff) return MA_ERR_ARG;
+    if (segments > 0x7fffffff) return kProbeErrArg;
     const bool need_a = mode == 0 || mode == 2 || mode == 3 || mode == 4;
     const bool need_b = mode == 3 || mode == 4, need_c = mode == 1 || mode == 2;
-    if ((need_a && !a) || (need_b && !b) || (need_c && !c) || (mode == 4 && !e)) return MA_ERR_ARG;
+    if ((need_a && !a) || (need_b && !b) || (need_c && !c) || (mode == 4 && !e)) return kProbeErrArg;
     const unsigned grid = (unsigned)(workgroups > 0 && workgroups < segments ? workgroups : segments);
     hipStream_t s = (hipStream_t)stream;
     switch (mode) {
@@ -97,5 +97,5 @@ extern "C" int ma_stream_probe(int mode, int nontemporal, int64_t bytes, int64_t
         case 3: return launch<3>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
         case 4: return launch<4>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
     }
-    return MA_ERR_ARG;
+    return kProbeErrArg;
 }

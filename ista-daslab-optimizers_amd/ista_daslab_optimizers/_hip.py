@@ -26,7 +26,8 @@ class MaTensor(ctypes.Structure):
                 ("min_vals", ctypes.c_void_p), ("max_vals", ctypes.c_void_p),
                 ("I", ctypes.c_void_p), ("V", ctypes.c_void_p), ("d", ctypes.c_int64),
                 ("k", ctypes.c_int64), ("lr", ctypes.c_double), ("weight_decay", ctypes.c_double),
-                ("index", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("index", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("quant_err", ctypes.c_void_p)]
 
 
 class MaHyper(ctypes.Structure):
@@ -82,7 +83,6 @@ def _load():
         "ma_sparse_linear_combination": (ci, [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp, ci,
                                               vp]),
         "ma_copy_values_typed": (ci, [i64, i64, i64, i64, vp, vp, vp, ci, ci, ci, vp]),
-        "ma_stream_probe": (ci, [ci, ci, i64, i64, vp, vp, vp, vp, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -100,7 +100,7 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_spanning_step", "ma_spanning_step_static", "ma_spanning_step_workspace",
            "ma_spanning_step_check", "ma_sparse_scalar_products",
            "ma_sparse_scalar_products_workspace", "ma_sparse_linear_combination",
-           "ma_copy_values_typed", "ma_stream_probe")
+           "ma_copy_values_typed")
 
 
 def error_string(code):

@@ -65,6 +65,8 @@ class _Table:
         self.view = np.frombuffer(self.records, dtype=_TENSOR_RECORD)
         for name in ('error', 'min_vals', 'max_vals', 'I', 'V'):
             self.view[name] = [e.st[name].data_ptr() for e in entries]
+        self.view['quant_err'] = [e.st['quant_err'].data_ptr() if 'quant_err' in e.st else 0
+                                  for e in entries]
         self.view['d'] = [e.st['d'] for e in entries]
         self.view['k'] = [e.st['k'] for e in entries]
 
@@ -191,6 +193,9 @@ class MicroAdam(torch.optim.Optimizer):
             self._check_param(p)
             self._initialize_parameter_state(p, lr, wd)
         repaired = self._repair_state(st)
+        if self.densify_update_using_quant_error and 'quant_err' not in st:
+            st['quant_err'] = torch.zeros_like(p)  # state loaded from a run with another alpha
+            repaired = True
         e = self._entries.get(p)
         if e is None or e.st is not st or repaired:
             e = self._entries[p] = _Entry(p, st, self._static_route(p, st))

@@ -416,7 +416,7 @@ static void clear(void *x, int64_t d, int dtype) {
  * double from the values as the buffer holds them (rounded to the gradient's type). */
 static int update_step_impl(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d,
                             int64_t *index, int16_t *I, uint16_t *V, uint8_t *error,
-                            uint16_t *min_vals, uint16_t *max_vals, double *mt) {
+                            uint16_t *min_vals, uint16_t *max_vals, double *mt, void *quant_err) {
     ora_geom g;
     if (h->alpha < 0 && h->alpha != -2.0) return -1;
     ora_geometry(d, h->max_d_block_size, h->k_init, h->q, &g);
@@ -442,24 +442,26 @@ static int update_step_impl(const ora_hyper *h, void *p, void *grad, int dtype, 
     /* :234-235 */
     if (h->wd > 0) ora_weight_decay(d, p, (float)(1.0 - h->lr * h->wd), dtype);
     /* :238-273, alpha == -2: p = p - a + Qinv(e_new).  The quant_err vector of :259-261, :271
-     * only feeds the logged norms. */
+     * (st['quant_err'], rewritten by every step) is kept in the caller's buffer if there is one. */
     if (h->alpha == -2.0) {
-        void *qe = NULL;
-        if (mt) { /* :259-261: quant_err = a (it has the parameter's type) */
+        void *qe = quant_err;
+        if (mt && !qe) {
             qe = malloc((size_t)d * 4);
             if (!qe) return -2;
-            memcpy(qe, grad, (size_t)d * (dtype == ORA_BF16 ? 2 : 4));
         }
+        /* :259-261: quant_err = a (it has the parameter's type) */
+        if (qe) memcpy(qe, grad, (size_t)d * (dtype == ORA_BF16 ? 2 : 4));
         ora_param_update(d, p, grad, -1.0f, dtype, dtype);                       /* STEP A, :264 */
         clear(grad, d, dtype);                                                   /* :267 */
         ora_asymm_block_quant_inv(d, h->q, error, min_vals, max_vals, grad, 1.0f, dtype);
         ora_param_update(d, p, grad, 1.0f, dtype, dtype);                        /* STEP B, :269 */
-        if (mt) { /* :271-273: quant_err -= Qinv(e_new), rounded to its type */
+        if (qe) /* :271: quant_err -= Qinv(e_new), rounded to its type */
             for (int64_t i = 0; i < d; ++i) st(qe, i, dtype, ld(qe, i, dtype) - ld(grad, i, dtype));
+        if (mt) { /* :272-273 */
             mt[0] += sum_squares(qe, d, dtype);
             mt[5] += count_zeros(qe, d, dtype);
-            free(qe);
         }
+        if (qe != quant_err) free(qe);
     }
     /* STEPS 10-11, :276-291 */
     clear(grad, d, dtype);
@@ -493,7 +495,18 @@ static int update_step_impl(const ora_hyper *h, void *p, void *grad, int dtype, 
 int ora_update_step(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d, int64_t *index,
                     int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
                     uint16_t *max_vals) {
-    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, NULL);
+    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, NULL,
+                            NULL);
+}
+
+/* ora_update_step / ora_step_metrics (metrics != NULL) that also keep st['quant_err']
+ * (micro_adam.py:67-68, :258-271; d elements of the parameter's type) when alpha == -2. */
+int ora_update_step_state(const ora_hyper *h, void *p, void *grad, int dtype, int64_t d,
+                          int64_t *index, int16_t *I, uint16_t *V, uint8_t *error,
+                          uint16_t *min_vals, uint16_t *max_vals, double *metrics,
+                          void *quant_err) {
+    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, metrics,
+                            quant_err);
 }
 
 /* A logging step (micro_adam.py:155-156, :271-272, :306-308, :320-324): ora_update_step, and
@@ -503,7 +516,8 @@ int ora_step_metrics(const ora_hyper *h, void *p, void *grad, int dtype, int64_t
                      int16_t *I, uint16_t *V, uint8_t *error, uint16_t *min_vals,
                      uint16_t *max_vals, double *metrics) {
     if (!metrics) return -1;
-    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, metrics);
+    return update_step_impl(h, p, grad, dtype, d, index, I, V, error, min_vals, max_vals, metrics,
+                            NULL);
 }
 
 /* ---- Sparse M-FAC's two window kernels (same I / V layout) ---------------- */

@@ -78,6 +78,8 @@ def lib():
         L.ora_update_step.restype = ci
         L.ora_step_metrics.argtypes = L.ora_update_step.argtypes + [ctypes.POINTER(f64)]
         L.ora_step_metrics.restype = ci
+        L.ora_update_step_state.argtypes = L.ora_step_metrics.argtypes + [vp]
+        L.ora_update_step_state.restype = ci
         L.ora_sparse_scalar_products.argtypes = [i64, i64, i64, i64, i64, vp, ci, vp, vp, ci, vp]
         L.ora_sparse_linear_combination.argtypes = [i64, i64, i64, i64, i64, vp, vp, vp, ci, vp,
                                                     ci]
@@ -251,6 +253,8 @@ class OracleMicroAdam:
         st["error"] = np.zeros(int(math.ceil(p.size / 2)), dtype=np.uint8)
         st["min_vals"] = np.zeros(g["stats_len"], dtype=np.uint16)
         st["max_vals"] = np.zeros(g["stats_len"], dtype=np.uint16)
+        if self.alpha == -2:  # micro_adam.py:67-68
+            st["quant_err"] = np.zeros_like(p)
         self.state[i] = st
         return st
 
@@ -275,7 +279,8 @@ class OracleMicroAdam:
             args = (ctypes.byref(h), _ptr(p), _ptr(g), dtype_tag(p), p.size, ctypes.byref(idx),
                     _ptr(st["I"]), _ptr(st["V"]), _ptr(st["error"]), _ptr(st["min_vals"]),
                     _ptr(st["max_vals"]))
-            rc = lib().ora_step_metrics(*args, sums) if metrics else lib().ora_update_step(*args)
+            qe = _ptr(st["quant_err"]) if "quant_err" in st else None
+            rc = lib().ora_update_step_state(*args, sums if metrics else None, qe)
             if rc != 0:
                 raise NotImplementedError("oracle covers alpha in [0, 1) and alpha == -2")
             st["index"] = idx.value

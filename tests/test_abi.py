@@ -32,9 +32,10 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header():
     from ista_daslab_optimizers import _hip
     # struct ma_tensor: 7 pointers, 2 int64, 2 double, 2 int32; struct ma_hyper: see header
-    assert ctypes.sizeof(_hip.MaTensor) == 7 * 8 + 2 * 8 + 2 * 8 + 2 * 4
+    assert ctypes.sizeof(_hip.MaTensor) == 7 * 8 + 2 * 8 + 2 * 8 + 2 * 4 + 8
     assert ctypes.sizeof(_hip.MaHyper) == 8 + 4 + 4 + 8 + 8 + 4 * 8
     assert _hip.MaTensor.lr.offset == 72 and _hip.MaTensor.index.offset == 88
+    assert _hip.MaTensor.quant_err.offset == 96
 
 
 def test_host_helpers_mirror_reference():

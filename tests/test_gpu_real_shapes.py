@@ -1,0 +1,87 @@
+"""The fused and spanning routes against the CPU oracle at real layer shapes of the three large
+benchmark lists (micro_adam.py:146-328 at the sizes where the hardware-sized block kernels run):
+
+  * Llama-2-7B: 4096 x 4096 and 11008 x 4096, q = 64, m = 10, k = 1 %: the 20480-element kernel
+    with the quantisation group compiled in, the hinted selection and the one-pass window stage;
+  * outlier 1.3B: 2048 x 8192 and 2048 x 6144 with the stress recipe (Student-t(3) x 1e-3, 1 % of
+    the rows x 100), q = 32, m = 20, k = 5 %, run past the step where all 20 rows are live and the
+    ring has wrapped: selection under skew, error-feedback range under outliers, the general
+    window stage with the window held in registers;
+  * Llama-3-8B: 4096 x 4096 and 1024 x 4096 with q = 100000 and alpha = 0.5: the two-pass route,
+    quantisation blocks that straddle 5-6 top-k blocks, the 2 x 16 table of the second pass.
+
+Gradients are drawn once per step from a seeded generator and the same bits go to the GPU
+optimizer and to the oracle.  Parameters are compared bit for bit after every step, the whole
+state (window as index sets with values, 4-bit codes, bf16 statistics) at the steps listed in
+each case.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import assert_state_equal, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _normal(shape, gen, std):
+    return (torch.randn(shape, generator=gen, device="cuda") * std).to(torch.bfloat16)
+
+
+def _outlier(shape, gen, hot_rows):
+    """Student-t with 3 degrees of freedom scaled by 1e-3, the rows in hot_rows times 100."""
+    z = torch.randn(shape, generator=gen, device="cuda")
+    chi = (torch.randn((3,) + tuple(shape), generator=gen, device="cuda") ** 2).sum(0) / 3
+    t = z / chi.sqrt() * 1e-3
+    t[hot_rows] *= 100
+    return t.to(torch.bfloat16)
+
+
+def _run(oracle, shapes, m, q, k_init, alpha, steps, full_at, route, kind):
+    from ista_daslab_optimizers import MicroAdam
+    gen = torch.Generator(device="cuda").manual_seed(2024)
+    start = [(torch.randn(s, generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+             for s in shapes]
+    hot = [torch.rand(s[0], generator=gen, device="cuda") < 0.01 for s in shapes]
+    oparams = [to_np(p).reshape(-1) for p in start]
+    oref = oracle.OracleMicroAdam(oparams, m, 1e-3, q, k_init, alpha, d_block_size=20480)
+    params = [torch.nn.Parameter(p.clone()) for p in start]
+    opt = MicroAdam(params, m=m, lr=1e-3, quant_block_size=q, k_init=k_init, alpha=alpha)
+    assert opt.d_block_size == 20480
+    for s in range(steps):
+        grads = [_outlier(shp, gen, h) if kind == "outlier" else _normal(shp, gen, 1e-3)
+                 for shp, h in zip(shapes, hot)]
+        host = [to_np(g).reshape(-1) for g in grads]
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+        assert all(opt._fusable(p, opt.state[p]) == route for p in params)
+        oref.step(host)
+        for i, p in enumerate(params):
+            ctx = f"{kind} step {s + 1} tensor {i} {tuple(shapes[i])}"
+            assert opt.state[p]["index"] == oref.state[i]["index"], ctx
+            got = to_np(p.data).reshape(-1)
+            if not np.array_equal(got, oparams[i]):
+                raise AssertionError(f"{ctx}: parameters differ at "
+                                     f"{int((got != oparams[i]).sum())} of {got.size} entries")
+            if s + 1 in full_at:
+                assert_state_equal(opt.state[p], oref.state[i], ctx)
+    return opt
+
+
+def test_llama2_7b_layers_match_oracle(oracle):
+    _run(oracle, [(4096, 4096), (11008, 4096)], 10, 64, 0.01, 0.0, 12, {1, 2, 10, 11, 12}, 1,
+         "normal")
+
+
+def test_outlier_layers_match_oracle_past_the_ring_wrap(oracle):
+    opt = _run(oracle, [(2048, 8192), (2048, 6144)], 20, 32, 0.05, 0.0, 23, {1, 2, 20, 21, 23}, 1,
+               "outlier")
+    # the data really are heavy-tailed: the largest window value dwarfs the typical one
+    V = opt.state[opt.param_groups[0]["params"][0]]["V"].float().abs()
+    assert float(V.max()) > 50 * float(V.median())
+
+
+def test_llama3_8b_layers_match_oracle(oracle):
+    _run(oracle, [(4096, 4096), (1024, 4096)], 10, 100000, 0.01, 0.5, 12, {1, 2, 10, 11, 12}, 2,
+         "normal")

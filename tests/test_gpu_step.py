@@ -6,6 +6,8 @@ min/max statistics, and here also the parameters themselves (the kernels use the
 unfused fp32 arithmetic as the oracle, so the stated 1e-3 / 1e-5 tolerance is met with
 zero difference; the tolerance check is kept as the documented bar).
 """
+import functools
+
 import numpy as np
 import pytest
 import torch
@@ -40,6 +42,9 @@ def _run(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused, gr
         for i, p in enumerate(gparams):
             ctx = f"step {s + 1} tensor {i} (d={sizes[i]})"
             assert_state_equal(opt.state[p], oref.state[i], ctx)
+            if alpha == -2:  # st['quant_err'] = a - Qinv(e_new), rewritten by every step
+                assert np.array_equal(to_np(opt.state[p]["quant_err"]).reshape(-1),
+                                      oref.state[i]["quant_err"]), f"{ctx}: quant_err"
             got, want = to_np(p.data), oparams[i]
             if not np.array_equal(got, want):
                 gf = oracle.bf16_to_f32(got) if got.dtype == np.uint16 else got
@@ -121,7 +126,8 @@ QUANT_ERR_CASES = [
 def test_step_quant_err_route(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused):
     opt = _run(oracle, sizes, dtype, m, q, k_init, alpha, wd, DB, steps, use_fused, zero_step=2,
                expect_route=use_fused)
-    assert all("quant_err" in st for st in opt.state.values())  # micro_adam.py:67-68
+    # micro_adam.py:67-68; _run has compared it with the oracle's after every step
+    assert all(st["quant_err"].any() for st in opt.state.values())
 
 
 SPANNING_CASES = [
@@ -540,52 +546,82 @@ def test_logged_sums_match_oracle(oracle, sizes, dtype, m, q, alpha, wd, route, 
             assert want["sparsity_u"] > 0
 
 
-@pytest.mark.parametrize("use_fused", [True, False], ids=["fused", "opbyop"])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_quantisation_rounding_boundaries(oracle, dtype, use_fused):
-    """The 4-bit codes where they are hardest to get right: every quantisation block holds its
-    minimum 0, its maximum M, and for each of the 15 rounding boundaries the value nearest to
-    (k + 1/2) u and its two neighbours (u = (M - 0) / 15 as the kernels form it), with M running
-    through bf16 significands and through every binary exponent from -126 to 126, so that steps u
-    that are subnormal, tiny, ordinary and huge all occur.  The fused kernels divide by a shared reciprocal where the
-    oracle divides; the codes must agree bit for bit all the same.  A second step with a zero
-    gradient dequantises and requantises them."""
-    from ista_daslab_optimizers import MicroAdam
-    q, DB = 64, 4096
+@functools.lru_cache(maxsize=None)
+def _boundary_gradient(dtype, q):
+    """Quantisation blocks of q elements that hold 0, M and the values around the rounding
+    boundaries (k + 1/2) M / 15, for M over bf16 significands x all binary exponents."""
     sig = [1.0, 1.0078125, 1.25, 1.5, 1.9921875, 1.328125, 1.7109375]
+    if q > 4096:
+        sig = [1.0, 1.5, 1.9921875]
     exps = list(range(-126, 127))
     gen = torch.Generator().manual_seed(17)
+    per_block = min(15, (q - 6) // 3)       # boundaries one block has room for
+    turns = [list(range(i, min(i + per_block, 15))) for i in range(0, 15, per_block)]
     blocks = []
     for e in exps:
         for s_ in sig:
             M = torch.tensor(s_ * 2.0 ** e, dtype=torch.float64).to(dtype)
             u = (M.float() - 0.0) / 15.0
-            vals = [torch.zeros((), dtype=dtype)] + [M] * 8
-            for k in range(15):
-                x = ((k + 0.5) * u.double()).to(dtype)
-                lo = torch.nextafter(x.float(), torch.tensor(0.0)).to(dtype) if dtype == torch.float32 \
-                    else (x.view(torch.int16) - 1).view(torch.bfloat16)
-                hi = torch.nextafter(x.float(), torch.tensor(float("inf"))).to(dtype) if dtype == torch.float32 \
-                    else (x.view(torch.int16) + 1).view(torch.bfloat16)
-                vals += [lo, x, hi]
-            rnd = (torch.rand(q - len(vals), generator=gen).double() * M.double()).to(dtype)
-            blk = torch.cat([torch.stack(vals), rnd])
-            blocks.append(blk[torch.randperm(q, generator=gen)])
-    g0 = torch.cat(blocks)
+            for ks in turns:
+                vals = [torch.zeros((), dtype=dtype)] + [M] * (8 if q >= 64 else 5)
+                for k in ks:
+                    x = ((k + 0.5) * u.double()).to(dtype)
+                    lo = torch.nextafter(x.float(), torch.tensor(0.0)).to(dtype) if dtype == torch.float32 \
+                        else (x.view(torch.int16) - 1).view(torch.bfloat16)
+                    hi = torch.nextafter(x.float(), torch.tensor(float("inf"))).to(dtype) if dtype == torch.float32 \
+                        else (x.view(torch.int16) + 1).view(torch.bfloat16)
+                    vals += [lo, x, hi]
+                rnd = (torch.rand(q - len(vals), generator=gen).double() * M.double()).to(dtype)
+                blk = torch.cat([torch.stack(vals), rnd])
+                blocks.append(blk[torch.randperm(q, generator=gen)])
+    return torch.cat(blocks)
+
+
+BOUNDARY_CASES = [
+    # DB, q, alpha, use_fused, route the tensor must take (0 op by op, 1 fused, 2 spanning,
+    # 3 fused densified)
+    (4096, 64, 0.0, True, 1),      # one-chunk kernel, quantisation group size at run time
+    (4096, 64, 0.0, False, 0),
+    (20480, 64, 0.0, True, 1),     # hardware block, group of 8 lanes compiled in, statistics
+    (20480, 32, 0.0, True, 1),     # shared across lanes; group of 4 lanes
+    (20480, 2048, 0.0, True, 1),   # quantisation blocks longer than a wave's stretch
+    (20480, 1024, 0.0, True, 1),
+    (20480, 64, 0.5, True, 3),     # both quantisations of the densified step
+    (20480, 2048, 0.5, True, 3),
+    (20480, 24576, 0.0, True, 2),  # two-pass route: statistics across top-k blocks
+    (20480, 24576, 0.5, True, 2),  # ... and the 2 x 16 table of its second pass
+]
+
+
+@pytest.mark.parametrize("DB,q,alpha,use_fused,route", BOUNDARY_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_quantisation_rounding_boundaries(oracle, dtype, DB, q, alpha, use_fused, route):
+    """The 4-bit codes where they are hardest to get right: every quantisation block holds its
+    minimum 0, its maximum M, and for the 15 rounding boundaries the value nearest to
+    (k + 1/2) u and its two neighbours (u = (M - 0) / 15 as the kernels form it; blocks too short
+    for all 15 take them in turns), with M running through bf16 significands and through every
+    binary exponent from -126 to 126, so that steps u that are subnormal, tiny, ordinary and huge
+    all occur.  The fused kernels divide by a shared reciprocal where the oracle divides; the
+    codes must agree bit for bit all the same, in every kernel instance that forms statistics or
+    codes in its own way.  A second step with a zero gradient dequantises and requantises them."""
+    from ista_daslab_optimizers import MicroAdam
+    g0 = _boundary_gradient(dtype, q)
     pad = (-g0.numel()) % DB
-    g0 = torch.cat([g0, torch.zeros(pad, dtype=dtype)])
+    if q <= DB:  # whole top-k blocks, so that the full-block kernel instances run
+        g0 = torch.cat([g0, torch.zeros(pad, dtype=dtype)])
     assert torch.isfinite(g0.float()).all()
     d = g0.numel()
     p0 = (torch.randn(d, generator=gen) * 0.02).to(dtype)
     oparams = [to_np(p0)]
-    oref = oracle.OracleMicroAdam(oparams, 4, 1e-3, q, 0.001, 0, d_block_size=DB)
+    oref = oracle.OracleMicroAdam(oparams, 4, 1e-3, q, 0.001, alpha, d_block_size=DB)
     gp = torch.nn.Parameter(p0.clone().cuda())
-    opt = MicroAdam([gp], m=4, lr=1e-3, quant_block_size=q, k_init=0.001)
+    opt = MicroAdam([gp], m=4, lr=1e-3, quant_block_size=q, k_init=0.001, alpha=alpha)
     opt.d_block_size = DB
     opt.use_fused = use_fused
     for step, g in enumerate([g0, torch.zeros_like(g0), g0]):
         gp.grad = g.clone().cuda()
         opt.step()
+        assert (opt._fusable(gp, opt.state[gp]) if use_fused else 0) == route
         oref.step([to_np(g)])
         assert_state_equal(opt.state[gp], oref.state[0], f"step {step + 1}")
         assert np.array_equal(to_np(gp.data), oparams[0]), f"step {step + 1}: parameters"

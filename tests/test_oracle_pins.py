@@ -366,6 +366,47 @@ def test_dense_limit_is_adam(oracle):
         assert np.allclose(p, tp.detach().numpy(), rtol=1e-5, atol=2e-7), t
 
 
+def test_window_ages_past_the_ring_wrap_follow_the_gradient_history(oracle):
+    """Which age a ring row gets once the ring has wrapped, pinned without the row formula:
+    with k_init = 1 every gradient is kept whole in the row its step wrote, so at step t the
+    update must be the sliding-window Adam direction over the last min(t, m) GRADIENTS, the
+    newest with weight beta^0 and the one from j steps ago with beta^j, whatever rows they
+    lie in.  A wrap in the wrong direction (ages counted from the wrong end of the ring, or an
+    off-by-one at the write slot) changes the weights of all rows and fails from t = m + 1 on.
+    t runs to 3 m + 2, three times round the ring."""
+    rng = np.random.default_rng(5)
+    d, m, lr, b1, b2, eps = 700, 5, 1e-2, 0.9, 0.999, 1e-8
+    p = (rng.standard_normal(d) * 0.1).astype(np.float32)
+    opt = oracle.OracleMicroAdam([p], m=m, lr=lr, quant_block_size=64, k_init=1.0,
+                                 d_block_size=256)
+    history = []
+    worst = 0.0
+    for t in range(1, 3 * m + 3):
+        g = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal(d).astype(np.float32)))
+        history.append(g.astype(np.float64))
+        before = p.astype(np.float64)
+        opt.step([g.copy()])
+        assert np.all(opt.state[0]["error"] == 0)
+        assert opt.state[0]["index"] == t % m
+        z1 = np.zeros(d)
+        z2 = np.zeros(d)
+        for j, gj in enumerate(reversed(history[-m:])):  # j steps ago
+            z1 += b1 ** j * gj
+            z2 += b2 ** j * gj ** 2
+        want = ((1 - b1) * z1 / (1 - b1 ** t)) / (eps + np.sqrt((1 - b2) * z2 / (1 - b2 ** t)))
+        got = (before - p.astype(np.float64)) / lr
+        # p is fp32 of size ~0.1 (ulp 7.5e-9), so a step's difference quotient carries ~1e-6
+        err = np.abs(got - want).max()
+        worst = max(worst, err)
+        assert err < 5e-6, (t, err)
+        # and the wrong direction is far outside that tolerance once the ring has wrapped
+        if t > m:
+            z1w = sum(b1 ** (m - 1 - j) * gj for j, gj in enumerate(reversed(history[-m:])))
+            wrong = ((1 - b1) * z1w / (1 - b1 ** t)) / (eps + np.sqrt((1 - b2) * z2 / (1 - b2 ** t)))
+            assert np.abs(wrong - want).max() > 1e-2
+    assert worst > 0.0
+
+
 # ---- parameter update ------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -429,6 +470,9 @@ def test_whole_step_matches_torch_restatement(oracle, sizes, dtype, m, q, k_init
             assert np.array_equal(bits(ts["min_vals"]), os_["min_vals"]), (s, i)
             assert np.array_equal(bits(ts["max_vals"]), os_["max_vals"]), (s, i)
             assert np.array_equal(bits(tref.params[i]), oparams[i]), (s, i)
+            if alpha == -2:  # st['quant_err'] = a - Qinv(e_new), micro_adam.py:258-271
+                assert np.array_equal(bits(ts["quant_err"]), os_["quant_err"]), (s, i)
+                assert os_["quant_err"].any()
 
 
 @pytest.mark.parametrize("sizes,dtype,m,q,k_init,alpha,wd,DB,steps", CASES)

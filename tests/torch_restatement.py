@@ -164,7 +164,7 @@ class TorchMicroAdam:
                 p.mul_(1 - lr * self.wd)
             if self.alpha == -2:
                 # micro_adam.py:258-273: p = p - a, then p = p + Qinv(e_new); quant_err = a - Qinv(e_new)
-                quant_err = torch.zeros_like(p).view(-1)
+                quant_err = st["quant_err"] = torch.zeros_like(p).view(-1)
                 quant_err.add_(grad)
                 p.add_(grad, alpha=-1)
                 grad.zero_()
