@@ -611,7 +611,7 @@ def test_quantisation_rounding_boundaries(oracle, dtype, DB, q, alpha, use_fused
         g0 = torch.cat([g0, torch.zeros(pad, dtype=dtype)])
     assert torch.isfinite(g0.float()).all()
     d = g0.numel()
-    p0 = (torch.randn(d, generator=gen) * 0.02).to(dtype)
+    p0 = (torch.randn(d, generator=torch.Generator().manual_seed(18)) * 0.02).to(dtype)
     oparams = [to_np(p0)]
     oref = oracle.OracleMicroAdam(oparams, 4, 1e-3, q, 0.001, alpha, d_block_size=DB)
     gp = torch.nn.Parameter(p0.clone().cuda())
