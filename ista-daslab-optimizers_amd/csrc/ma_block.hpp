@@ -80,6 +80,8 @@ struct FusedParams {
     float keep;       // (float)(1 - alpha): share that stays in the error feedback
     // logging steps (kernels compiled with kAuxLog): kMetricSlots floats per work item
     float *metrics;
+    // the block kernel ends with the quantisation; window_param_kernel does the rest
+    int32_t win_apart;
 };
 
 // Extras of a block kernel (template parameter AUX, a set of bits).  Kernels with extras run
@@ -185,9 +187,7 @@ __device__ __forceinline__ BlockGeo make_geo(const FusedParams &P, int ti, int64
 // which of them they fill and which they consume.
 //   FULL: the block has exactly kRound*C elements, so no chunk needs a bounds check.
 //   QL:   lanes per quantisation block fixed at compile time (4: q = 32, 8: q = 64), 0: any.
-//   HOLD: the general window stage may keep the block's window entries in registers (40 of
-//         them), for kernels compiled with the register budget of two workgroups per CU.
-template <class R, bool FULL, int QL, bool HOLD = false, int AUX = 0>
+template <class R, bool FULL, int QL, int AUX = 0>
 struct FusedBlock {
     typedef typename R::elem_t elem_t;
     static constexpr int C = R::kC;
@@ -269,11 +269,6 @@ struct FusedBlock {
     bool row_in_lds;  // the window row of this step is taken from sel_idx / sel_val, not from HBM
     Divisor d15;
 
-    // window entries of the block, two per register as they lie in memory (index pairs in
-    // hI, value pairs in hV): step s = (row, trip) holds pair trip * kWG + tid of the row
-    static constexpr int kHold = HOLD ? 20 : 1;
-    uint32_t hI[kHold], hV[kHold];   //                      load_held          -> update
-    bool holding;
     RawChunk<R> praw[C];          // parameters              load_params_window -> update
     uint32_t entI[kEnt];          // entries of the older window rows, kept as loaded so that
     uint32_t entV[kEnt];          // nothing waits for them    load_params_window -> update
@@ -310,7 +305,6 @@ struct FusedBlock {
         d15.r = 0x1.111112p-4f;
         slot_clear = false;
         row_in_lds = true;
-        holding = false;
         wide = false;
         if constexpr (LOG) {
 #pragma unroll
@@ -353,116 +347,6 @@ struct FusedBlock {
                     const int64_t at = (int64_t)row * G.D.k + G.col0 + (e - row * G.kb);
                     entI[i] = reinterpret_cast<const uint16_t *>(G.D.I)[at];
                     entV[i] = G.D.V[at];
-                }
-            }
-        }
-    }
-
-    // ---- the whole window of the block into registers, for the general window stage
-    // Entries travel two per 32-bit load (from any 2-byte boundary), so a row of the block has
-    // to hold an even number of entries; otherwise, or when the window has more than kHold
-    // steps, the stage streams the entries as window_accumulate does.
-    __device__ __forceinline__ bool can_hold(const BlockGeo &G) const {
-        const int pairs = G.kb >> 1;
-        const int trips = (pairs + kWG - 1) / kWG;
-        return HOLD && P.L.cell_bytes == 0 && (G.kb & 1) == 0 && P.W.rows * trips <= kHold;
-    }
-
-    // current == false: the older rows, from memory (can be asked for before the selection);
-    // current == true: the row this step selected, from LDS
-    __device__ __forceinline__ void load_held(const BlockGeo &G, bool current) {
-        if (!current) holding = can_hold(G);
-        if (!holding) return;
-        const int pairs = G.kb >> 1;
-        const int trips = (pairs + kWG - 1) / kWG;
-        // (a pair may start on any 2-byte boundary: the hardware takes unaligned loads)
-        struct __attribute__((packed, aligned(2))) Pair {
-            uint32_t w;
-        };
-        const int16_t *Ib = G.D.I + G.col0;
-        const uint16_t *Vb = G.D.V + G.col0;
-        int row = 0, it = 0;  // uniform
-#pragma unroll
-        for (int s = 0; s < kHold; ++s) {
-            if (!current) {
-                hI[s] = 0xffffffffu;  // index 0xffff lies in no range
-                hV[s] = 0;
-            }
-            if (row < P.W.rows) {
-                const int w = it * kWG + tid;
-                if (w < pairs) {
-                    const bool from_lds = row == G.D.row && row_in_lds;
-                    if (current && from_lds) {
-                        hI[s] = reinterpret_cast<const uint32_t *>(sel_idx)[w];
-                        hV[s] = reinterpret_cast<const uint32_t *>(sel_val)[w];
-                    } else if (!current && !from_lds) {
-                        const int64_t at = (int64_t)row * G.D.k + 2 * w;
-                        hI[s] = reinterpret_cast<const Pair *>(Ib + at)->w;
-                        hV[s] = reinterpret_cast<const Pair *>(Vb + at)->w;
-                    }
-                }
-                if (++it == trips) {
-                    it = 0;
-                    ++row;
-                }
-            }
-        }
-    }
-
-    // window_accumulate from the held entries: same order of additions (rows in increasing
-    // order, a barrier after each row; the two entries of a register are distinct coordinates)
-    __device__ __forceinline__ void accumulate_held(int kb, int lo, int hi) {
-        for (int i = tid; i < hi - lo; i += kWG) {
-            z1[i] = 0.0f;
-            z2[i] = 0.0f;
-        }
-        __syncthreads();
-        const int trips = ((kb >> 1) + kWG - 1) / kWG;
-        const uint32_t span = (uint32_t)(hi - lo);
-        // lane l keeps the weights of row l (a window has at most 64 rows), handed out by
-        // readlane: no memory access per step
-        const float w1v = P.W.w1[lane], w2v = P.W.w2[lane];
-        int row = 0, it = 0;  // uniform
-#pragma unroll
-        for (int s = 0; s < kHold; ++s) {
-            if (row < P.W.rows) {
-                const uint32_t c0 = (hI[s] & 0xffffu) - (uint32_t)lo, c1 = (hI[s] >> 16) - (uint32_t)lo;
-                // rows written by these kernels are in increasing coordinate order, so a range
-                // is a stretch of lanes: most waves have nothing to add and skip the rest
-                if (__builtin_amdgcn_ballot_w64(c0 < span || c1 < span) != 0) {
-                    const uint32_t b0 = hV[s] & 0xffffu, b1 = hV[s] >> 16;
-                    const bool ok0 = c0 < span && (b0 & 0x7fffu) != 0;
-                    const bool ok1 = c1 < span && (b1 & 0x7fffu) != 0;
-                    const float w1 =
-                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w1v), row));
-                    const float w2 =
-                        __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w2v), row));
-                    const float v0 = bf2f(b0), v1 = bf2f(b1);
-                    const float a10 = w1 * v0, a11 = w1 * v1;
-                    const float q0 = v0 * v0, q1 = v1 * v1;
-                    const float a20 = w2 * q0, a21 = w2 * q1;
-                    float r10 = 0.0f, r20 = 0.0f, r11 = 0.0f, r21 = 0.0f;
-                    if (ok0) {
-                        r10 = z1[c0];
-                        r20 = z2[c0];
-                    }
-                    if (ok1) {
-                        r11 = z1[c1];
-                        r21 = z2[c1];
-                    }
-                    if (ok0) {
-                        z1[c0] = r10 + a10;
-                        z2[c0] = r20 + a20;
-                    }
-                    if (ok1) {
-                        z1[c1] = r11 + a11;
-                        z2[c1] = r21 + a21;
-                    }
-                }
-                if (++it == trips) {
-                    it = 0;
-                    ++row;
-                    __syncthreads();
                 }
             }
         }
@@ -992,7 +876,7 @@ struct FusedBlock {
         for (int j = 0; j < kOwned; ++j) {
             upd[j] = 0xffffffffu;
             if (own[j] != 0xffffffffu) {
-                const float u = adam_direction(z1[j], z2[j], P.W.s1, P.W.s2, P.W.eps);
+                const float u = adam_update<R::kBF16>(z1[j], z2[j], P.W.s1, P.W.s2, P.W.eps);
                 upd[j] = own[j] | f2bf(u) << 16;
             }
         }
@@ -1054,14 +938,11 @@ struct FusedBlock {
         __syncthreads();  // the LDS of the selection is reused below
         for (int lo = 0; lo < n; lo += P.L.sub_len) {
             const int hi = lo + P.L.sub_len < n ? lo + P.L.sub_len : n;
-            if (HOLD && holding)
-                accumulate_held(G.kb, lo, hi);
-            else
-                window_accumulate(wv, G.kb, lo, hi, z1, z2);
+            window_accumulate(wv, G.kb, lo, hi, z1, z2);
             for (int c = tid; c < hi - lo; c += kWG) {
                 float u = 0.0f;
                 if (z1[c] != 0.0f || z2[c] != 0.0f)
-                    u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                    u = adam_update<R::kBF16>(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
                 z1[c] = R::kBF16 ? bf2f(f2bf(u)) : u;
             }
             __syncthreads();
@@ -1169,7 +1050,7 @@ struct FusedBlock {
                             const float vv = v * v;
                             const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
                             const float u =
-                                adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                                adam_update<R::kBF16>(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
                             cell16[idx] = (uint16_t)f2bf(u);
                         } else {
                             multi |= 1u << i;
@@ -1206,7 +1087,7 @@ struct FusedBlock {
                 }
                 const int used = (int)(*mcount < (uint32_t)cap ? *mcount : (uint32_t)cap);
                 for (int sl = tid; sl < used; sl += kWG) {
-                    const float u = adam_direction(s1[sl], s2[sl], P.W.s1, P.W.s2, P.W.eps);
+                    const float u = adam_update<R::kBF16>(s1[sl], s2[sl], P.W.s1, P.W.s2, P.W.eps);
                     cell16[scoord[sl]] = (uint16_t)f2bf(u);
                 }
                 __syncthreads();
@@ -1224,7 +1105,7 @@ struct FusedBlock {
                     const float a2 = __uint_as_float(sh[kShW2 + row]) * vv;
                     if (mask == 1u << row) {
                         const float u =
-                            adam_direction(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
+                            adam_update<R::kBF16>(0.0f + a1, 0.0f + a2, P.W.s1, P.W.s2, P.W.eps);
                         if (R::kBF16) {
                             cell16[idx] = (uint16_t)f2bf(u);
                         } else {  // fp32: the update keeps its bits in a record of its own,
@@ -1274,7 +1155,7 @@ struct FusedBlock {
                         s1 = s1 + f1[o];
                         s2 = s2 + f2[o];
                     }
-                    const float u = adam_direction(s1, s2, P.W.s1, P.W.s2, P.W.eps);
+                    const float u = adam_update<R::kBF16>(s1, s2, P.W.s1, P.W.s2, P.W.eps);
                     if (R::kBF16) {
                         cell16[idx] = (uint16_t)f2bf(u);
                     } else {  // the owner's record has given its sums and takes the update
@@ -1300,7 +1181,7 @@ struct FusedBlock {
                 window_accumulate(wv, kb, lo, hi, z1, z2);
                 for (int c = tid; c < hi - lo; c += kWG) {
                     if (z1[c] != 0.0f || z2[c] != 0.0f) {
-                        const float u = adam_direction(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
+                        const float u = adam_update<R::kBF16>(z1[c], z2[c], P.W.s1, P.W.s2, P.W.eps);
                         if (R::kBF16) cell16[lo + c] = (uint16_t)f2bf(u);
                         else cell32[lo + c] = __float_as_uint(u);
                     }
@@ -1972,7 +1853,12 @@ __device__ __forceinline__ int find_tensor(const FusedParams &P, int w) {
 
 // One workgroup per block: any block shape.  Tensor i contributes its blocks
 // blk0 .. blk0 + (first_block[i+1] - first_block[i]) - 1.
-template <class R, int MIN_WAVES, int QL, bool DENSE = false, bool HOLD = false, int AUX = 0>
+//   WIN: what becomes of the window and the parameters.  kWinFused: everything in this kernel.
+//        kWinApart: nothing; the kernel ends with the quantisation, and window_param_kernel,
+//        launched behind it, forms the update and steps the parameters.
+constexpr int kWinFused = 0, kWinApart = 2;
+
+template <class R, int MIN_WAVES, int QL, bool DENSE = false, int WIN = kWinFused, int AUX = 0>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int item = xcd_contiguous_item(P.total_items);
@@ -1981,8 +1867,6 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
     auto run = [&](auto &fb) {
         fb.load_grad_inputs(G);
         fb.dequant(G);
-        // the older window rows are most of this path's traffic: asked for before the selection
-        if constexpr (HOLD) fb.load_held(G, false);
         fb.topk_and_row(G);
         if constexpr (DENSE) {
             fb.quantize_dense(G);
@@ -1993,18 +1877,17 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         } else {
             // parameters and window entries are asked for before the quantisation, which
             // hides their latency (the selection runs with more registers free without them)
-            fb.load_params_window(G);
+            if constexpr (WIN != kWinApart) fb.load_params_window(G);
             fb.quantize(G);
-            if constexpr (HOLD) fb.load_held(G, true);
-            fb.update(G);
+            if constexpr (WIN != kWinApart) fb.update(G);
         }
         fb.log_flush(item, 0xffu);
     };
     if (G.n == R::kC * kRound) {
-        FusedBlock<R, true, QL, HOLD, AUX> fb(P, lds);
+        FusedBlock<R, true, QL, AUX> fb(P, lds);
         run(fb);
     } else {
-        FusedBlock<R, false, QL, HOLD, AUX> fb(P, lds);
+        FusedBlock<R, false, QL, AUX> fb(P, lds);
         run(fb);
     }
 }
@@ -2058,11 +1941,280 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
                                        : 1u << kMtError);
     };
     if (G.n == R::kC * kRound) {
-        FusedBlock<R, true, 0, false, AUX> fb(P, lds);
+        FusedBlock<R, true, 0, AUX> fb(P, lds);
         run(fb);
     } else {
-        FusedBlock<R, false, 0, false, AUX> fb(P, lds);
+        FusedBlock<R, false, 0, AUX> fb(P, lds);
         run(fb);
+    }
+}
+
+
+// =============================================================================================
+// Window and parameters apart from the block kernel (kWinApart): Adam direction from the window
+// (MA:277-291), p = p * (1 - lr*wd) (MA:234-235), p += -lr * u (MA:304), for windows with about
+// as many entries as the block has coordinates (m = 20 rows of 5 %), where the sums of all
+// coordinates do not fit the LDS at once and the block kernel's own window stage is a chain of
+// barrier-separated row steps.  One workgroup per top-k block; it reads the window rows
+// (including the one the block kernel has just written) and the parameters, nothing else.
+//
+// Rows that list their entries by increasing coordinate (as every kernel of this library writes
+// them when a block row has more than 512 entries) are cut at the multiples of 1024
+// coordinates: chunk ch of a row is the stretch table[row][ch] .. table[row][ch + 1] of its
+// entries.  A wave then owns a chunk: its 1024 pairs of sums live in the wave's own 8 KiB of
+// LDS, it adds the rows' stretches in row order (the LDS operations of one wave execute in
+// program order and a row names a coordinate once, so no barrier is needed and every sum is
+// formed in row order, as compute_microadam_update forms it), and lane l steps the 16
+// parameters at 16 l of the chunk.
+// A block in which some row is not in increasing order, or holds an index outside the block,
+// takes the general form instead: coordinate ranges of 4096 with a barrier after every row.
+//   LDS: the kSh* words | table: rows x (chunks + 1) int32 at L.off_slot, row stride
+//   L.slot_cells | sums: 8 x (kWinChunk + 8) pairs of floats at L.off_union (per wave one
+//   cell (z1, z2) per coordinate of a chunk and a spare one; the general form uses the same
+//   memory as 2 x 4096 floats).
+// =============================================================================================
+constexpr int kWinShift = 9;
+constexpr int kWinChunk = 1 << kWinShift;  // coordinates per chunk: 8 for each of 64 lanes
+constexpr int kWinRowBatch = 10;    // rows whose stretches are requested together
+
+// two window entries as they lie in memory, from any 2-byte boundary (the hardware takes
+// unaligned loads)
+struct __attribute__((packed, aligned(2))) EntryPair {
+    uint32_t w;
+};
+
+// value of the lane below (lane 0 and lanes without a source get `first`)
+__device__ __forceinline__ uint32_t lane_below(uint32_t v, uint32_t first) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xF,
+                                                 0xF, false);
+}
+
+template <class R, int MIN_WAVES>
+__global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParams P) {
+    typedef typename R::elem_t elem_t;
+    extern __shared__ __align__(16) unsigned char lds[];
+    uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
+    int *table = reinterpret_cast<int *>(lds + P.L.off_slot);
+    float *sums = reinterpret_cast<float *>(lds + P.L.off_union);
+    const int item = xcd_contiguous_item(P.total_items);
+    const int ti = find_tensor(P, item);
+    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = G.n, kb = G.kb, rows = P.W.rows;
+    const int nch = (n + kWinChunk - 1) / kWinChunk;
+    const int stride = nch + 1;
+    const int64_t k = G.D.k;
+    const uint16_t *Ib = reinterpret_cast<const uint16_t *>(G.D.I) + G.col0;
+    const uint16_t *Vb = G.D.V + G.col0;
+    elem_t *p = reinterpret_cast<elem_t *>(G.D.p) + G.e0;
+    const float neg_lr = G.D.neg_lr, decay = G.D.decay;
+    const bool apply_decay = G.D.apply_decay != 0;
+
+    // ---- where every row crosses the chunk boundaries, and whether all rows are in order.
+    //      Thread t takes the entries 2t and 2t + 1 of every row (one load), the entry before
+    //      them comes from the lane below, for lane 0 from memory.
+    if (tid == 0) sh[0] = 0;
+    for (int i = tid; i < rows * stride; i += kWG) table[i] = 2 * kb;
+    __syncthreads();
+    bool bad = false;
+    for (int j0 = 0; j0 < kb; j0 += 2 * kWG) {
+        const int j = j0 + 2 * tid;
+        for (int r0 = 0; r0 < rows; r0 += kWinRowBatch) {
+            uint32_t pair[kWinRowBatch], before[kWinRowBatch];
+#pragma unroll
+            for (int i = 0; i < kWinRowBatch; ++i) {
+                pair[i] = 0xffffffffu;
+                before[i] = 0;
+                if (r0 + i < rows) {
+                    const uint16_t *Ir = Ib + (int64_t)(r0 + i) * k;
+                    if (j + 1 < kb)
+                        pair[i] = reinterpret_cast<const EntryPair *>(Ir + (unsigned)j)->w;
+                    else if (j < kb)
+                        pair[i] = (uint32_t)Ir[(unsigned)j] | 0xffff0000u;
+                    if (lane == 0 && j > 0 && j < kb) before[i] = Ir[(unsigned)(j - 1)];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kWinRowBatch; ++i) {
+                if (r0 + i < rows) {
+                    // (the lane below holds the two entries before this lane's)
+                    const uint32_t below = lane_below(pair[i] >> 16, before[i]);
+                    const int c0 = (int)(pair[i] & 0xffffu), c1 = (int)(pair[i] >> 16);
+                    const int cb = j > 0 ? (int)below : -1;
+                    int *trow = table + (r0 + i) * stride;
+                    if (j < kb) {
+                        if (c0 <= cb || c0 >= n) {
+                            bad = true;
+                        } else {
+                            for (int ch = (cb >> kWinShift) + 1; ch <= (c0 >> kWinShift); ++ch)
+                                trow[ch] = 2 * j;
+                        }
+                    }
+                    if (j + 1 < kb) {
+                        if (c1 <= c0 || c1 >= n) {
+                            bad = true;
+                        } else {
+                            for (int ch = (c0 >> kWinShift) + 1; ch <= (c1 >> kWinShift); ++ch)
+                                trow[ch] = 2 * (j + 1);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    if (bad) atomicOr(&sh[0], 1u);
+    __syncthreads();
+    const bool in_order = sh[0] == 0;
+    // table[row][ch]: byte offset of the first entry of chunk ch in the row's stretch of the
+    // block
+
+    // p = p * decay; p += -lr * u for the 8 parameters at `off`, u from their 8 pairs of sums
+    auto step8 = [&](int off, const RawChunk<R> &praw, const float (&a1)[8], const float (&a2)[8]) {
+        float pv[8];
+        praw.to_float(pv);
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+            float u = 0.0f;
+            if (a1[e] != 0.0f || a2[e] != 0.0f) {
+                u = adam_update<R::kBF16>(a1[e], a2[e], P.W.s1, P.W.s2, P.W.eps);
+            }
+            if (apply_decay) {
+                pv[e] = pv[e] * decay;
+                if (R::kBF16) pv[e] = bf2f(f2bf(pv[e]));
+            }
+            const float prod = neg_lr * u;
+            pv[e] = pv[e] + prod;
+        }
+        store8(p, off, n, true, pv);
+    };
+
+    if (in_order) {
+        // per wave one cell (z1, z2) per coordinate of a chunk and a spare one that takes what
+        // is not for this chunk
+        constexpr int kPerLane = kWinChunk / kWave;  // coordinates of a chunk per lane
+        float2 *z = reinterpret_cast<float2 *>(sums) + wave * (kWinChunk + 8);
+        const uint32_t lane2 = (uint32_t)lane * 2u;
+        for (int ch = wave; ch < nch; ch += kWaves) {
+            const int base = ch * kWinChunk, off = base + lane * kPerLane;
+            RawChunk<R> praw[kPerLane / kChunk];
+#pragma unroll
+            for (int h = 0; h < kPerLane / kChunk; ++h)
+                praw[h].load(p, off + h * kChunk, n, base + kWinChunk <= n);
+            const float4 zero4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+            for (int i = 0; i < kPerLane / 2; ++i)
+                reinterpret_cast<float4 *>(z + lane * kPerLane)[i] = zero4;
+            __builtin_amdgcn_wave_barrier();
+            for (int r0 = 0; r0 < rows; r0 += kWinRowBatch) {
+                // ---- all requests of the batch first: entry s + lane of every row's stretch.
+                //      Entries past the stretch (they belong to later chunks) or past the row
+                //      (the buffer returns index 0, value 0 for them) are sorted out when they
+                //      are added.  A batch that reaches past the last live row reads those rows
+                //      through buffers of no bytes, with weights 0: straight-line code, so that
+                //      nothing between the requests waits for an answer.
+                uint32_t ei[kWinRowBatch], ev[kWinRowBatch];
+                float w1[kWinRowBatch], w2[kWinRowBatch];
+                uint32_t longer = 0;  // bit i: row r0 + i has more than 64 entries in the chunk
+                const int *tp = table + r0 * stride + ch;
+#pragma unroll
+                for (int i = 0; i < kWinRowBatch; ++i) {
+                    const bool live = r0 + i < rows;
+                    const int r = live ? r0 + i : 0;
+                    w1[i] = live ? P.W.w1[r] : 0.0f;
+                    w2[i] = live ? P.W.w2[r] : 0.0f;
+                    const uint32_t at = (uint32_t)tp[i * stride] + lane2;
+                    const uint32_t e2 = (uint32_t)tp[i * stride + 1];
+                    if (live && __builtin_amdgcn_ballot_w64(at + 2u * kWave < e2) != 0)
+                        longer |= 1u << i;
+                    const uint32_t bytes = live ? 2u * (uint32_t)kb : 0u;
+                    const __amdgpu_buffer_rsrc_t bi = byte_buffer(Ib + (int64_t)r * k, bytes);
+                    const __amdgpu_buffer_rsrc_t bv = byte_buffer(Vb + (int64_t)r * k, bytes);
+                    ei[i] = __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at, 0, 0);
+                    ev[i] = __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at, 0, 0);
+                }
+                // ---- then the sums, row after row.  An entry of a later chunk goes to the
+                //      spare cell; one past the row (index 0, value 0) adds 0 to the first cell
+                //      or goes there too; +-0 values change nothing anywhere (the rows of a fresh window
+                //      are all (0, 0), and a coordinate counts as named when a sum is not zero).
+#pragma unroll
+                for (int i = 0; i < kWinRowBatch; ++i) {
+                    auto add = [&](uint32_t idx, uint32_t vb) {
+                        const uint32_t c = min(idx - (uint32_t)base, (uint32_t)kWinChunk);
+                        const float v = bf2f(vb);
+                        const float t1 = w1[i] * v;
+                        const float vv = v * v;
+                        const float t2 = w2[i] * vv;
+                        float2 x = z[c];
+                        x.x = x.x + t1;
+                        x.y = x.y + t2;
+                        z[c] = x;
+                    };
+                    add(ei[i], ev[i]);
+                    if ((longer >> i) & 1u) {  // the rest of the stretch, before the next row
+                        const int r = r0 + i;
+                        const uint32_t s2 = (uint32_t)tp[i * stride];
+                        const uint32_t e2 = (uint32_t)tp[i * stride + 1];
+                        const __amdgpu_buffer_rsrc_t bi =
+                            byte_buffer(Ib + (int64_t)r * k, 2u * (uint32_t)kb);
+                        const __amdgpu_buffer_rsrc_t bv =
+                            byte_buffer(Vb + (int64_t)r * k, 2u * (uint32_t)kb);
+                        for (uint32_t a2 = s2 + 2u * kWave; a2 < e2; a2 += 2u * kWave) {
+                            const uint32_t at = a2 + lane2;
+                            const uint32_t idx =
+                                __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at, 0, 0);
+                            const uint32_t vb =
+                                __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at, 0, 0);
+                            add(idx, vb);
+                        }
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int h = 0; h < kPerLane / kChunk; ++h) {
+                float a1[8], a2[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 q =
+                        reinterpret_cast<const float4 *>(z + lane * kPerLane + h * kChunk)[i];
+                    a1[2 * i] = q.x;
+                    a2[2 * i] = q.y;
+                    a1[2 * i + 1] = q.z;
+                    a2[2 * i + 1] = q.w;
+                }
+                if (off + h * kChunk < n) step8(off + h * kChunk, praw[h], a1, a2);
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else {
+        constexpr int kRange = 4096;
+        float *z1 = sums, *z2 = sums + kRange;
+        WindowView wv;
+        wv.I = G.D.I + G.col0;
+        wv.V = Vb;
+        wv.k = k;
+        wv.rows = rows;
+        wv.cur_row = -1;
+        wv.cur_idx = nullptr;
+        wv.cur_val = nullptr;
+        wv.w1 = P.W.w1;
+        wv.w2 = P.W.w2;
+        for (int lo = 0; lo < n; lo += kRange) {
+            const int hi = lo + kRange < n ? lo + kRange : n;
+            window_accumulate(wv, kb, lo, hi, z1, z2);
+            for (int off = lo + tid * kChunk; off < hi; off += kWG * kChunk) {
+                RawChunk<R> praw;
+                praw.load(p, off, n, false);
+                float a1[8], a2[8];
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    a1[e] = off + e < hi ? z1[off - lo + e] : 0.0f;
+                    a2[e] = off + e < hi ? z2[off - lo + e] : 0.0f;
+                }
+                step8(off, praw, a1, a2);
+            }
+            __syncthreads();
+        }
     }
 }
 
@@ -2083,17 +2235,16 @@ static int allow_big_lds(K kernel, int bytes) {
 constexpr int kWavesThreeWG = 3 * kWG / 256;  // three workgroups per CU
 constexpr int kMinWaves = kWG / 128;  // waves per SIMD the block kernels are compiled for: two workgroups per CU
 
-template <class R, int QL, bool DENSE = false, bool HOLD = false, int AUX = 0>
+template <class R, int QL, bool DENSE = false, int WIN = kWinFused, int AUX = 0>
 static int launch_fused_one(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // bf16 blocks of up to 20480 elements fit 80 registers and a third of the LDS: three
-    // workgroups per CU; the general window stage with the window held in registers, and the
-    // kernels with extras, take the budget of two
+    // workgroups per CU; the kernels with extras take the budget of two
     constexpr int kWaves_ =
-        (R::kBF16 && R::kC <= kClass2 && !HOLD && AUX == 0) ? kWavesThreeWG : kMinWaves;
+        (R::kBF16 && R::kC <= kClass2 && AUX == 0) ? kWavesThreeWG : kMinWaves;
     // grid == 0: the preparation of the launch only (whatever may fail apart from the launch
     // itself), so that a call can prepare all its launches before the first one starts
-    if (grid == 0) return allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, lds_bytes);
-    return launch_kernel(fused_step_kernel<R, kWaves_, QL, DENSE, HOLD, AUX>, dim3(grid), kWG,
+    if (grid == 0) return allow_big_lds(fused_step_kernel<R, kWaves_, QL, DENSE, WIN, AUX>, lds_bytes);
+    return launch_kernel(fused_step_kernel<R, kWaves_, QL, DENSE, WIN, AUX>, dim3(grid), kWG,
                          lds_bytes, s, P);
 }
 
@@ -2102,10 +2253,10 @@ template <template <int> class RT, bool DENSE, int AUX>
 static int launch_fused_aux(int C, unsigned grid, int lds_bytes, hipStream_t s,
                             const FusedParams &P) {
     switch (C) {
-        case kClass0: return launch_fused_one<RT<kClass0>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
-        case kClass1: return launch_fused_one<RT<kClass1>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
-        case kClass2: return launch_fused_one<RT<kClass2>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
-        case kClass3: return launch_fused_one<RT<kClass3>, 0, DENSE, false, AUX>(grid, lds_bytes, s, P);
+        case kClass0: return launch_fused_one<RT<kClass0>, 0, DENSE, kWinFused, AUX>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0, DENSE, kWinFused, AUX>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0, DENSE, kWinFused, AUX>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0, DENSE, kWinFused, AUX>(grid, lds_bytes, s, P);
     }
     return MA_ERR_BLOCK_SIZE;
 }
@@ -2127,16 +2278,32 @@ static int launch_fused_dense(int C, unsigned grid, int lds_bytes, hipStream_t s
     return MA_ERR_BLOCK_SIZE;
 }
 
+// the block kernels that leave window and parameters to window_param_kernel
+template <template <int> class RT>
+static int launch_fused_apart(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                              const FusedParams &P) {
+    if (C == kClass2 && P.q_shift == 6)
+        return launch_fused_one<RT<kClass2>, 8, false, kWinApart>(grid, lds_bytes, s, P);
+    if (C == kClass2 && P.q_shift == 5)
+        return launch_fused_one<RT<kClass2>, 4, false, kWinApart>(grid, lds_bytes, s, P);
+    switch (C) {
+        case kClass0: return launch_fused_one<RT<kClass0>, 0, false, kWinApart>(grid, lds_bytes, s, P);
+        case kClass1: return launch_fused_one<RT<kClass1>, 0, false, kWinApart>(grid, lds_bytes, s, P);
+        case kClass2: return launch_fused_one<RT<kClass2>, 0, false, kWinApart>(grid, lds_bytes, s, P);
+        case kClass3: return launch_fused_one<RT<kClass3>, 0, false, kWinApart>(grid, lds_bytes, s, P);
+    }
+    return MA_ERR_BLOCK_SIZE;
+}
+
+template <class R>
+static int launch_window_param(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
+    if (grid == 0) return allow_big_lds(window_param_kernel<R, kWavesThreeWG>, lds_bytes);
+    return launch_kernel(window_param_kernel<R, kWavesThreeWG>, dim3(grid), kWG, lds_bytes, s, P);
+}
+
 template <template <int> class RT>
 static int launch_fused(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P) {
     // the hardware-sized block gets kernels with the quantisation group size compiled in
-    if constexpr (RT<kClass2>::kBF16) {
-        // windows too large for the one-pass stage: the general stage, window in registers
-        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 6)
-            return launch_fused_one<RT<kClass2>, 8, false, true>(grid, lds_bytes, s, P);
-        if (C == kClass2 && P.L.cell_bytes == 0 && P.q_shift == 5)
-            return launch_fused_one<RT<kClass2>, 4, false, true>(grid, lds_bytes, s, P);
-    }
     if (C == kClass2 && P.q_shift == 6) return launch_fused_one<RT<kClass2>, 8>(grid, lds_bytes, s, P);
     if (C == kClass2 && P.q_shift == 5) return launch_fused_one<RT<kClass2>, 4>(grid, lds_bytes, s, P);
     switch (C) {
@@ -2186,6 +2353,12 @@ static int launch_span(int C, int pass, unsigned grid, int lds_bytes, hipStream_
 // The instantiations, one translation unit each.
 int launch_fused_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
 int launch_fused_f32(int C, unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
+int launch_fused_apart_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                            const FusedParams &P);
+int launch_fused_apart_f32(int C, unsigned grid, int lds_bytes, hipStream_t s,
+                           const FusedParams &P);
+int launch_window_param_bf16(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
+int launch_window_param_f32(unsigned grid, int lds_bytes, hipStream_t s, const FusedParams &P);
 int launch_fused_dense_bf16(int C, unsigned grid, int lds_bytes, hipStream_t s,
                             const FusedParams &P);
 int launch_fused_dense_f32(int C, unsigned grid, int lds_bytes, hipStream_t s,

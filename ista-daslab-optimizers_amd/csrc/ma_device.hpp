@@ -1049,4 +1049,42 @@ __device__ __forceinline__ float adam_direction(float z1, float z2, float s1, fl
     return mh / (eps + sqrtf(vh));
 }
 
+// The same direction for a bf16 update: only its rounding to bf16 is wanted, so eight bits of
+// the quotient decide and an approximation settles almost every case.  q = mh * rcp(eps +
+// sqrt(vh)) with the hardware's square root and reciprocal (one ulp each) lies within 3.5 * 2^-23
+// (relative; at most 7 ulp) of the correctly rounded quotient of the correctly rounded terms,
+// provided nothing on the way is subnormal or overflows: vh >= 2^-100 (then the root and the
+// denominator are comfortably normal) and q itself has an exponent in [-100, 100].  Then q and
+// the exact quotient round to the same bf16 value unless q lies within 7 ulp of a tie, i.e.
+// unless its low 16 bits are that close to 0x8000; 16 is asked.  A wave in which some lane fails
+// one of the tests (about one call in thirty at random data) takes the exact way for all lanes.
+// Returns the update as bf16 bits.
+__device__ __forceinline__ uint32_t adam_direction_bf16(float z1, float z2, float s1, float s2,
+                                                        float eps) {
+    const float mh = z1 * s1;
+    const float vh = z2 * s2;
+    const float root = __builtin_amdgcn_sqrtf(vh);
+    const float den = eps + root;
+    const float q = mh * __builtin_amdgcn_rcpf(den);
+    const uint32_t b = __float_as_uint(q);
+    // low 16 bits outside [0x8000 - 15, 0x8000 + 15]
+    const bool far_from_tie = (b & 0xffffu) - 0x7ff1u > 30u;
+    const bool safe = vh >= 0x1p-100f && ((b >> 23) & 0xffu) - 27u <= 200u && far_from_tie;
+    if (__builtin_amdgcn_ballot_w64(!safe) == 0) return f2bf(q);
+    return f2bf(adam_direction(z1, z2, s1, s2, eps));
+}
+
+// The direction as the update buffer of the data's type holds it: rounded to bf16 for bf16 data
+// (so that a later conversion to bf16 changes nothing), fp32 otherwise.
+template <bool BF16>
+__device__ __forceinline__ float adam_update(float z1, float z2, float s1, float s2, float eps) {
+    if (BF16) return bf2f(adam_direction_bf16(z1, z2, s1, s2, eps));
+    return adam_direction(z1, z2, s1, s2, eps);
+}
+
+// A raw buffer over `bytes` bytes at p: loads past the end return 0 instead of faulting.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t byte_buffer(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+
 }  // namespace ma

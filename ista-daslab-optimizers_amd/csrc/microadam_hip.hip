@@ -290,7 +290,8 @@ __global__ __launch_bounds__(kWG) void window_update_kernel(int64_t d, int dbs, 
         window_accumulate(wv, kb, lo, hi, z1, z2);
         for (int c = tid; c < hi - lo; c += kWG)
             if (z1[c] != 0.0f || z2[c] != 0.0f)
-                stf(out, e0 + lo + c, adam_direction(z1[c], z2[c], W.s1, W.s2, W.eps));
+                stf(out, e0 + lo + c,
+                    adam_update<sizeof(T) == 2>(z1[c], z2[c], W.s1, W.s2, W.eps));
         __syncthreads();
     }
 }
@@ -357,6 +358,36 @@ static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_
     }
     const int zbytes = L.z_cap * (L.fast_cap ? 16 : 8);
     L.total = L.off_union + align16(zbytes > kHistBytes ? zbytes : kHistBytes);
+    return L;
+}
+
+// LDS plan of a block kernel that ends with the quantisation: the selection's needs only (the
+// cells are where the fast selection parks the block; longer block rows take the general
+// selection, which leaves the block in registers).
+static LdsMap plan_lds_select_only(int dbs_max, int kb_max) {
+    LdsMap L;
+    memset(&L, 0, sizeof L);
+    L.off_sel_idx = kMiscBytes;
+    L.off_sel_val = L.off_sel_idx + align16(kb_max * 2);
+    L.off_slot = L.off_sel_val + align16(kb_max * 2);
+    L.slot_cells = (dbs_max + 7) & ~7;
+    L.cell_bytes = 2;
+    L.off_union = L.off_slot + (kb_max <= kWG ? align16(L.slot_cells * 2) : 0);
+    L.hist_log2 = 5;
+    L.total = L.off_union + kHistBytes;
+    return L;
+}
+
+// LDS plan of window_param_kernel: the chunk table of every row, then 8192 floats of sums.
+static LdsMap plan_lds_window_param(int dbs_max, int m) {
+    LdsMap L;
+    memset(&L, 0, sizeof L);
+    L.off_slot = kMiscBytes;
+    L.slot_cells = (dbs_max + kWinChunk - 1) / kWinChunk + 1;
+    L.off_union = L.off_slot + align16(m * L.slot_cells * 4);  // (a batch may read, and ignore,
+                                                               // table rows past the last: they
+                                                               // lie in the sums)
+    L.total = L.off_union + kWaves * (kWinChunk + 8) * 8;  // (above the general form's 32 KiB)
     return L;
 }
 
@@ -677,7 +708,9 @@ int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
 struct PlannedLaunch {
     FusedParams P;
     int C;
+    int kind;  // kWholeStep, or the two launches that share a step: kBlockPart, kWindowPart
 };
+enum { kWholeStep = 0, kBlockPart = 1, kWindowPart = 2 };
 
 // Short tensors (one block of up to 4096 / 12288 elements) have kernels of their own, so that
 // they do not occupy a workgroup sized for the hardware block; but when a call holds few of
@@ -795,11 +828,26 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.alpha = (float)alpha;
             P.keep = (float)(1.0 - alpha);
             P.metrics = (aux & kAuxLog) ? metrics + items_before * kMetricSlots : nullptr;
+            P.win_apart = 0;
+            plan.back().kind = kWholeStep;
+            int rc = P.L.total > kLdsLimit ? MA_ERR_LDS : 0;
+            if (!span && !dense && !aux && P.L.cell_bytes == 0) {
+                // a window too large for the one-pass stage: the block kernel ends with the
+                // quantisation, a second launch over the same blocks forms the update
+                P.win_apart = 1;
+                P.L = plan_lds_select_only(dbs_max, kb_max);
+                plan.back().kind = kBlockPart;
+                PlannedLaunch second = plan.back();
+                second.kind = kWindowPart;
+                second.P.L = plan_lds_window_param(dbs_max, h->m);
+                if (second.P.L.total > kLdsLimit || P.L.total > kLdsLimit) rc = MA_ERR_LDS;
+                plan.push_back(second);
+            }
             items_before += items;
             count = 0;
             items = 0;
             dbs_max = kb_max = 0;
-            return P.L.total > kLdsLimit ? MA_ERR_LDS : 0;
+            return rc;
         };
         for (int i = 0; i < n_tensors; ++i) {
             const ma_tensor &t = tensors[i];
@@ -862,6 +910,12 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
         } else if (!span && aux) {
             rc = bf16 ? launch_fused_aux_bf16(L.C, aux, grid, P.L.total, s, P)
                       : launch_fused_aux_f32(L.C, aux, grid, P.L.total, s, P);
+        } else if (L.kind == kWindowPart) {
+            rc = bf16 ? launch_window_param_bf16(grid, P.L.total, s, P)
+                      : launch_window_param_f32(grid, P.L.total, s, P);
+        } else if (L.kind == kBlockPart) {
+            rc = bf16 ? launch_fused_apart_bf16(L.C, grid, P.L.total, s, P)
+                      : launch_fused_apart_f32(L.C, grid, P.L.total, s, P);
         } else if (!span) {
             rc = bf16 ? launch_fused_bf16(L.C, grid, P.L.total, s, P)
                       : launch_fused_f32(L.C, grid, P.L.total, s, P);

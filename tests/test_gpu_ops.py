@@ -216,6 +216,35 @@ def test_compute_microadam_update(ext, oracle, dtype, m, dbs, kb, nblocks, tail,
     assert np.array_equal(to_np(out), oout)
 
 
+@pytest.mark.parametrize("eps", [1e-8, 0.0, 1e-30, 1.0])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_direction_over_many_magnitudes(ext, oracle, dtype, eps):
+    """The direction (z1 s1) / (eps + sqrt(z2 s2)) of compute_microadam_update
+    (micro_adam.py:277-291) on 4 million coordinates whose window values run over 30 decades, down
+    to values whose squares are subnormal or vanish, every coordinate named by all three rows (so
+    the sums cancel to all sizes).  For bf16 updates the kernels settle the rounding from an
+    approximate quotient and take the exactly rounded way only near a tie: the bits must be the
+    oracle's (correctly rounded square root and division) everywhere all the same."""
+    _, ma = ext
+    rng = np.random.default_rng(123)
+    m, dbs, nblocks, t = 3, 4096, 1024, 7
+    d = k = nblocks * dbs
+    I = np.stack([np.tile(rng.permutation(dbs).astype(np.int16), nblocks) for _ in range(m)])
+    mag = 10.0 ** rng.uniform(-24, 6, size=(m, k))
+    mag[:, : k // 8] = 10.0 ** rng.uniform(-3, -1, size=(m, k // 8))   # ordinary gradients
+    val = (mag * rng.choice([-1.0, 1.0], size=(m, k))).astype(np.float32)
+    val[0, k // 8: k // 4] = -val[1, k // 8: k // 4]                    # sums that nearly cancel
+    V = oracle.f32_to_bf16(val.reshape(-1)).reshape(m, k)
+    out = torch.zeros(d, dtype=dtype, device="cuda")
+    oout = to_np(torch.zeros(d, dtype=dtype))
+    ma.compute_microadam_update(1, 512, 100, t, 0.9, 0.999, eps, dbs, dbs, d, m, k,
+                                torch.from_numpy(I).cuda(), to_torch(V.reshape(-1)).view(m, k), out)
+    oracle.compute_microadam_update(t, 0.9, 0.999, eps, dbs, dbs, d, m, k, I, V, oout)
+    got = to_np(out)
+    bad = np.nonzero(got != oout)[0]
+    assert bad.size == 0, (bad.size, bad[:5], got[bad[:5]], oout[bad[:5]])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("d", [8192, 1001, 5])
 def test_param_update(hip, oracle, dtype, d):
