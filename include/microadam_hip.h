@@ -42,7 +42,7 @@ extern "C" {
 
 #define MA_MAX_WINDOW 64 /* largest window length m the kernels take */
 #define MA_MAX_D_BLOCK 32768
-#define MA_STATIC_WORKSPACE_BYTES (8 << 20) /* scratch ma_spanning_step_static holds per GPU */
+#define MA_STATIC_WORKSPACE_BYTES (16 << 20) /* scratch ma_spanning_step_static holds per GPU */
 #define MA_MAX_SPARSE_ROWS 4096 /* most window rows the Sparse M-FAC kernels take */
 
 const char *ma_error_string(int code);
@@ -176,16 +176,23 @@ int ma_fused_step_densified(const ma_tensor *tensors /* host */, int n_tensors,
 
 /* The whole of update_step (MA:146-328) when the quantisation blocks are at least as long as
  * the top-k blocks (the reference's documented setting is quant_block_size = 100000), for
- * alpha == 0 and for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), in two
- * passes per top-k block:
- *   1. a = g + Qinv(e); block top-k -> I[index], V[index]; the residual r is written over g
- *      (the reference's step destroys p.grad as well, MA:190-316) and its min / max per block
- *      to the workspace;
+ * alpha == 0 and for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316).  A
+ * quantisation block then covers several top-k blocks, whose workgroups have to exchange the
+ * extremes of the residual (through the workspace) before any of them can form codes:
+ *   1. a = g + Qinv(e); block top-k -> I[index], V[index]; min / max of the residual r per
+ *      top-k block to the workspace;
  *   2. min / max of r per quantisation block from the workspace; e1 = Q(r);
  *      alpha == 0: error = e1, min_vals, max_vals; window -> Adam direction; p update (with
  *      decoupled weight decay);
  *      alpha > 0: Qinv(e1) stays in registers; window -> Adam direction, + alpha * Qinv(e1);
  *      p update; error = Q((1 - alpha) * Qinv(e1)), min_vals, max_vals.
+ * With alpha > 0 these are two kernel passes and r travels from the first to the second in g.
+ * With alpha == 0 they are one pass: a workgroup publishes its extremes and takes those of its
+ * neighbours as they arrive; it waits for them a bounded time only (MA_SPAN_SPIN_LIMIT polls
+ * per neighbour, an environment variable, default 256, 0 = no wait), and a block that gives
+ * up leaves r in g and is taken through step 2 by a second launch.  Either way g may hold r
+ * instead of the gradient afterwards (the reference's step destroys p.grad as well,
+ * MA:190-316).
  * The caller advances st['index'] itself.  Conditions (else MA_ERR_NOT_FUSABLE, nothing
  * launched): 0 <= alpha < 1 (MA:18); quant_block_size a multiple of 8, not below
  * min(d, d_block_size), below 2^30 and covering at most 62 top-k blocks; alignment as for
@@ -196,7 +203,7 @@ int ma_spanning_step(const ma_tensor *tensors /* host */, int n_tensors,
                       const ma_hyper *hyper /* host */, double alpha, void *workspace,
                       int64_t workspace_bytes, void *stream);
 
-/* Bytes of workspace ma_spanning_step needs for this list (16 per top-k block); -1 on bad
+/* Bytes of workspace ma_spanning_step needs for this list (32 per top-k block); -1 on bad
  * arguments.  Host-only. */
 int64_t ma_spanning_step_workspace(const ma_tensor *tensors /* host */, int n_tensors,
                                     const ma_hyper *hyper /* host */);
@@ -206,16 +213,22 @@ int ma_spanning_step_check(const ma_tensor *tensor /* host */, const ma_hyper *h
                             double alpha);
 
 /* ma_spanning_step for callers that cannot allocate device memory or hand over a workspace
- * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * (tight serving loops, harnesses that forbid hipMalloc, code under HIP graph capture).  No
  * counterpart in the reference.  Same arguments, conditions and results as ma_spanning_step;
- * the per-block extremes of the residual go to a fixed array of MA_STATIC_WORKSPACE_BYTES
- * (8 MiB) that the library holds in the memory of every GPU it runs on until the process ends,
- * which is room for 524 288 top-k blocks per call (10.7e9 elements at d_block_size 20480); a
- * list that needs more is rejected with MA_ERR_WORKSPACE and nothing is launched.  The call
- * allocates and frees nothing.  The array's address is looked up at the first call on each
- * device.  All calls on one GPU share that GPU's array: it need not be cleared between calls
- * (the first pass writes every entry the second pass reads), but calls whose kernels may
- * overlap on one GPU (different streams) race on it. */
+ * the workspace is a fixed array of MA_STATIC_WORKSPACE_BYTES (16 MiB) that the library holds
+ * in the memory of every GPU it runs on until the process ends, which is room for 524 288
+ * top-k blocks per call (10.7e9 elements at d_block_size 20480; the Llama-3-8B list needs
+ * 12.6 MB); a list that needs more is rejected with MA_ERR_WORKSPACE and nothing is launched.
+ * The call allocates and frees no device memory (on the host it builds its launch plan in
+ * ordinary heap memory, as every step entry point does).  The array's address is looked up at
+ * the first call on each device, for the device that is current then: the current device must
+ * be the one `stream` belongs to.  All calls on one GPU share that GPU's array: it need not be
+ * cleared between calls (a call clears or overwrites what it reads), but calls whose kernels
+ * may overlap on one GPU (different streams) race on it.  Under graph capture: the step
+ * number, the ring row and the learning rate travel by value in the kernel arguments, so a
+ * captured call replays exactly that step; capture it anew (or update the kernel nodes) for
+ * every step, and make the first, uncaptured call on the device before capturing (it looks up
+ * the array and sets kernel attributes). */
 int ma_spanning_step_static(const ma_tensor *tensors /* host */, int n_tensors,
                              const ma_hyper *hyper /* host */, double alpha, void *stream);
 

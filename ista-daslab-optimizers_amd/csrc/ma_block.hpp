@@ -82,6 +82,9 @@ struct FusedParams {
     float *metrics;
     // the block kernel ends with the quantisation; window_param_kernel does the rest
     int32_t win_apart;
+    // one-pass form of the two-pass route: polls a workgroup spends at most on waiting for the
+    // extremes of the blocks that share its quantisation blocks (0: it does not wait at all)
+    int32_t spin_limit;
 };
 
 // Extras of a block kernel (template parameter AUX, a set of bits).  Kernels with extras run
@@ -97,6 +100,7 @@ struct FusedParams {
 //            straight into the parameters, p = p - a, then p = p + Qinv(e) (each rounded to
 //            the parameter's type) before the Adam step.
 constexpr int kAuxLog = 1, kAuxQuantErr = 2;
+constexpr int kSpanWords = 8;  // workspace words per top-k block of the two-pass route
 constexpr int kMetricSlots = 8;
 enum { kMtQuantErr = 0, kMtGrad = 1, kMtUpdate = 2, kMtError = 3, kMtUpdateZeros = 4, kMtQuantErrZeros = 5 };
 
@@ -1394,7 +1398,21 @@ struct FusedBlock {
     // statistics of r2 over a quantisation block are r2 at the codes of r's extremes: pass 2
     // needs no second reduction across blocks.
     // Segment 0 of a block is its part in the quantisation block of its first element,
-    // segment 1 the rest.  Workspace: 4 floats (min0, max0, min1, max1) per block.
+    // segment 1 the rest.  Workspace: a slot of 8 words per block: min0, max0, min1, max1
+    // (floats), then four words the one-pass form uses for its list of deferred blocks.
+    //
+    // One-pass form (the same arithmetic, the residual never leaves the registers; the
+    // workspace starts with the four floats of every block as all-ones words and the rest
+    // zero): a workgroup publishes the extremes of its block right after the selection, goes
+    // on with what does not need the statistics, and then takes the extremes of the blocks
+    // that share its quantisation blocks as they are published.  Blocks that share a quantisation block are
+    // neighbours, neighbouring blocks are dispatched together, and every workgroup publishes
+    // before it waits, so the wait is short; it is bounded all the same (spin_limit polls), and
+    // a workgroup that gives up stores its residual in the gradient buffer and lists its block:
+    // a second launch takes the listed blocks through the second pass of the two-pass form.
+    // The old statistics of a quantisation block are overwritten by the block that holds its
+    // first element only after that block has seen all blocks of the quantisation block
+    // published, i.e. after all of them have read the old statistics.
     // =========================================================================================
     struct Span {
         int64_t qb0;  // quantisation block of the block's first element
@@ -1443,7 +1461,7 @@ struct FusedBlock {
                                                    float (&mx)[2]) {
         wg_minmax2(mn, mx);
         if (tid == 0)
-            *reinterpret_cast<float4 *>(G.D.ws + block_id(G) * 4) =
+            *reinterpret_cast<float4 *>(G.D.ws + block_id(G) * kSpanWords) =
                 make_float4(mn[0], mx[0], mn[1], mx[1]);
     }
 
@@ -1466,7 +1484,7 @@ struct FusedBlock {
                 const int64_t b = b_lo + lane;
                 if (b <= b_hi) {
                     const int seg = b * dbs >= first ? 0 : 1;
-                    const float *w = G.D.ws + b * 4 + seg * 2;
+                    const float *w = G.D.ws + b * kSpanWords + seg * 2;
                     mn = w[0];
                     mx = w[1];
                 }
@@ -1483,6 +1501,12 @@ struct FusedBlock {
     __device__ __forceinline__ void span_statistics(const BlockGeo &G, const Span &S) {
         float mnx[2], mxx[2];
         gather_extremes(G, S, mnx, mxx);
+        statistics_from_extremes<DENSE>(mnx, mxx);
+    }
+
+    template <bool DENSE>
+    __device__ __forceinline__ void statistics_from_extremes(const float (&mnx)[2],
+                                                             const float (&mxx)[2]) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             sp_mn[s2] = f2bf(mnx[s2]);
@@ -1505,6 +1529,14 @@ struct FusedBlock {
             hi = P.keep * hi;
             sp2_mn[s2] = f2bf(to_elem(0.0f + lo));
             sp2_mx[s2] = f2bf(to_elem(0.0f + hi));
+        }
+        // (the same in every lane: kept in scalar registers from here on)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            sp_mn[s2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)sp_mn[s2]);
+            sp_mx[s2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)sp_mx[s2]);
+            sp2_mn[s2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)sp2_mn[s2]);
+            sp2_mx[s2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)sp2_mx[s2]);
         }
     }
 
@@ -1664,6 +1696,143 @@ struct FusedBlock {
         store_partials(G, mn, mx);
     }
 
+    // ---- one-pass form ---------------------------------------------------------------------
+    // extremes of the residual (in the registers) per segment, to the workspace, then the flag
+    __device__ __forceinline__ void span_publish(const BlockGeo &G, const Span &S) {
+        const int n = FULL ? C * kRound : G.n;
+        float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float x[8];
+                float lmn = INFINITY, lmx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+                if (FULL) {
+                    minmax8(x, lmn, lmx);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < kChunk; ++e) {
+                        if (off + e < n) {
+                            lmn = fmin_raw(lmn, x[e]);
+                            lmx = fmax_raw(lmx, x[e]);
+                        }
+                    }
+                }
+                const bool second = off >= S.bnd;
+                mn[0] = fmin_raw(mn[0], second ? INFINITY : lmn);
+                mx[0] = fmax_raw(mx[0], second ? -INFINITY : lmx);
+                mn[1] = fmin_raw(mn[1], second ? lmn : INFINITY);
+                mx[1] = fmax_raw(mx[1], second ? lmx : -INFINITY);
+            }
+        }
+        wg_minmax2(mn, mx);
+        if (tid == 0) {
+            // One 64-bit store per segment, past this XCD's L2 (device scope) and without any
+            // fence: the pair is all that is handed over, it arrives whole, and a pair that
+            // has not arrived reads as the all-ones words the workspace was cleared to (a
+            // published minimum is never that NaN; a block whose extremes are NaN looks
+            // unpublished, and its neighbours give up and take the second pass).
+            uint64_t *w = reinterpret_cast<uint64_t *>(G.D.ws + block_id(G) * kSpanWords);
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+                __hip_atomic_store(w + s2,
+                                   (uint64_t)__float_as_uint(mn[s2]) |
+                                       (uint64_t)__float_as_uint(mx[s2]) << 32,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+
+    // Waits (wave 0 polls, at most P.spin_limit times per flag) until all blocks that share
+    // this block's quantisation blocks have published, then forms the statistics as
+    // span_statistics does.  False, for every thread, if some block did not publish in time.
+    // Uses sh[kShTies] and the 4 words at sh[kShSel]; two barriers.
+    template <bool DENSE>
+    __device__ __forceinline__ bool span_await(const BlockGeo &G, const Span &S) {
+        const int64_t q = P.q_span;
+        const int64_t dbs = G.D.d < P.d_block_size ? G.D.d : P.d_block_size;
+        const int64_t nblk = (G.D.d + dbs - 1) / dbs;
+        if (wave == 0) {
+            bool ok = true;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                float mn = INFINITY, mx = -INFINITY;
+                if (s2 == 0 || S.bnd != 0x7fffffff) {
+                    const int64_t Q = S.qb0 + s2;
+                    const int64_t first = Q * q;
+                    const int64_t b_lo = first / dbs;
+                    int64_t b_hi = (first + q - 1) / dbs;
+                    b_hi = b_hi < nblk - 1 ? b_hi : nblk - 1;
+                    const int64_t b = b_lo + lane;
+                    if (b <= b_hi) {
+                        const int seg = b * dbs >= first ? 0 : 1;
+                        uint64_t *w =
+                            reinterpret_cast<uint64_t *>(G.D.ws + b * kSpanWords) + seg;
+                        int left = P.spin_limit;
+                        uint64_t pair =
+                            __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        while ((uint32_t)pair == 0xffffffffu && left > 0) {
+                            __builtin_amdgcn_s_sleep(8);
+                            --left;
+                            pair = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                        ok = ok && (uint32_t)pair != 0xffffffffu;
+                        mn = __uint_as_float((uint32_t)pair);
+                        mx = __uint_as_float((uint32_t)(pair >> 32));
+                    }
+                    group_minmax<0>(mn, mx, kWave);
+                }
+                if (lane == 0) {
+                    sh[kShSel + 2 * s2] = __float_as_uint(mn);
+                    sh[kShSel + 2 * s2 + 1] = __float_as_uint(mx);
+                }
+            }
+            const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+            if (lane == 0) sh[kShTies] = all_ok ? 1u : 0u;
+        }
+        __syncthreads();
+        const bool all_ok = sh[kShTies] != 0;
+        float mnx[2], mxx[2];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            mnx[s2] = __uint_as_float(sh[kShSel + 2 * s2]);
+            mxx[s2] = __uint_as_float(sh[kShSel + 2 * s2 + 1]);
+        }
+        __syncthreads();  // the words are free again
+        if (all_ok) statistics_from_extremes<DENSE>(mnx, mxx);
+        return all_ok;
+    }
+
+    // Gives up on the one-pass form for this block: the residual goes to the gradient buffer,
+    // where the second pass of the two-pass form expects it.
+    __device__ __forceinline__ void span_defer(const BlockGeo &G) {
+        const int n = FULL ? C * kRound : G.n;
+        elem_t *out = reinterpret_cast<elem_t *>(const_cast<void *>(G.D.g)) + G.e0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int off = chunk_off<C>(wave, c, lane);
+            if (FULL || off < n) {
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+                store8(out, off, FULL ? 0x7fffffff : n, true, x);
+            }
+        }
+    }
+
+    // the residual of chunk c as fp32: from the registers of the one-pass form, or as the
+    // second pass loaded it
+    template <bool FROM_R>
+    __device__ __forceinline__ void residual8(int c, float (&x)[8]) const {
+        if (FROM_R) {
+#pragma unroll
+            for (int e = 0; e < kChunk; ++e) x[e] = r.val(c, e);
+        } else {
+            graw[c].to_float(x);
+        }
+    }
+
     // ---- pass 2 -----------------------------------------------------------------------
     // The window row the first pass wrote comes back into sel_idx / sel_val, where the window
     // stages expect the row of this step: requested first, stored once the other requests
@@ -1700,6 +1869,7 @@ struct FusedBlock {
     }
 
     // alpha == 0, second pass: e = Q(r) against the statistics of r, and the statistics arrays
+    template <bool FROM_R = false>
     __device__ __forceinline__ void span_codes_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
@@ -1712,7 +1882,7 @@ struct FusedBlock {
             if (FULL || off < n) {
                 const bool second = off >= S.bnd;
                 float x[8], cf[8];
-                graw[c].to_float(x);
+                residual8<FROM_R>(c, x);
                 codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
                 log_error(cf, second ? mn1 : mn0, second ? u1 : u0, FULL ? kChunk : n - off);
 #pragma unroll
@@ -1750,6 +1920,7 @@ struct FusedBlock {
     // d1 = Qinv(e1) takes 16 values per segment, and alpha * d1 and the code of r2 with them:
     // both come from a table of 2 x 16 entries that 32 threads fill first, so that an element
     // costs one quantisation, not two.
+    template <bool FROM_R = false>
     __device__ __forceinline__ void span_param_stage(const BlockGeo &G, const Span &S) {
         const int n = FULL ? C * kRound : G.n;
         const TensorDesc &D = G.D;
@@ -1785,7 +1956,7 @@ struct FusedBlock {
             if (FULL || off < n) {
                 const bool second = off >= S.bnd;
                 float x[8], cf[8];
-                graw[c].to_float(x);
+                residual8<FROM_R>(c, x);
                 codes8(x, second ? mn1 : mn0, second ? u1 : u0, cf);
                 const uint2 *mine = table + (second ? 16 : 0);
                 float pv[8], uv[8];
@@ -1898,13 +2069,33 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
 //               statistics), PASS 3 (codes of the residual)
 //   Logging steps: the first pass leaves |g|^2 (and, as PASS 4, the update's sums) and clears
 //   the components no pass forms; the second leaves the rest.
+// One-pass form of the same route, alpha == 0, no logging: PASS 6 does the whole step of a block,
+// exchanging the extremes of the residual through the workspace; PASS 8 is PASS 3 for the blocks
+// PASS 6 deferred, launched behind it with a fixed number of workgroups.  The deferred blocks are
+// listed: their count is word kSpanDeferCount of the first block slot of the launch's workspace
+// (the slot of block 0 of the launch's first tensor), the i-th deferred work item is word
+// kSpanDeferItem of the i-th slot from there (the launch has at most as many work items as
+// there are slots from its first to the end of the workspace).
+// (With alpha > 0 the one-pass form was built as well and measured slower than the two passes:
+// its second half needs the registers of the second pass on top of the residual, which costs
+// the third workgroup per CU or spills, and neither pass is short of memory bandwidth by
+// enough to pay for that.)
+constexpr int kSpanDeferItem = 4, kSpanDeferCount = 6;
+
 template <class R, int MIN_WAVES, int PASS, int AUX = 0>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
-    const int item = xcd_contiguous_item(P.total_items);
-    const int ti = find_tensor(P, item);
-    const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
-    auto run = [&](auto &fb) {
+    constexpr bool kSweep = PASS == 8;
+    uint32_t *slots = reinterpret_cast<uint32_t *>(P.t[0].ws);
+    uint32_t *defer_count = slots + kSpanDeferCount;
+    // (PASS 6) this block gives up: listed for the sweep
+    auto list_deferred = [&](int item) {
+        if (threadIdx.x == 0) {
+            const uint32_t at = atomicAdd(defer_count, 1u);
+            slots[(int64_t)at * kSpanWords + kSpanDeferItem] = (uint32_t)item;
+        }
+    };
+    auto run = [&](auto &fb, const BlockGeo &G, int item) {
         const auto S = fb.make_span(G);
         if constexpr (PASS == 1 || PASS == 4) {
             fb.span_load_grad_inputs(G, S);
@@ -1928,10 +2119,28 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             // last in the stage below, so they are the ones that wait)
             fb.load_params(G);
             fb.span_param_stage(G, S);
-        } else {
+        } else if constexpr (PASS == 3 || PASS == 8) {
             fb.span_load_residual(G);
             fb.template span_statistics<false>(G, S);
             fb.span_codes_stage(G, S);
+        } else {  // PASS 6
+            fb.span_load_grad_inputs(G, S);
+            fb.span_dequant(G, S);
+            fb.topk_and_row(G);
+            fb.span_publish(G, S);
+            // (the parameters are asked for once the residual has left the registers: both
+            // held through the wait and the codes would not fit the register budget of three
+            // workgroups per CU)
+            fb.wide = fb.wide_window(G);
+            if (fb.wide) fb.load_window_wide(G); else fb.load_window(G);
+            if (fb.template span_await<false>(G, S)) {
+                fb.template span_codes_stage<true>(G, S);
+            } else {
+                fb.span_defer(G);
+                list_deferred(item);
+            }
+            fb.load_params(G);
+            fb.update(G);
         }
         constexpr unsigned kUnused = 1u << kMtQuantErr | 1u << kMtQuantErrZeros | 3u << 6;
         constexpr unsigned kUpdate = 1u << kMtUpdate | 1u << kMtUpdateZeros;
@@ -1940,15 +2149,29 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
                            : PASS == 2 ? kUpdate | 1u << kMtError
                                        : 1u << kMtError);
     };
-    if (G.n == R::kC * kRound) {
-        FusedBlock<R, true, 0, AUX> fb(P, lds);
-        run(fb);
+    auto one = [&](int item) {
+        const int ti = find_tensor(P, item);
+        const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
+        if (G.n == R::kC * kRound) {
+            FusedBlock<R, true, 0, AUX> fb(P, lds);
+            run(fb, G, item);
+        } else {
+            FusedBlock<R, false, 0, AUX> fb(P, lds);
+            run(fb, G, item);
+        }
+    };
+    if constexpr (kSweep) {
+        const uint32_t listed = *defer_count < (uint32_t)P.total_items ? *defer_count
+                                                                       : (uint32_t)P.total_items;
+        for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
+            const uint32_t item = slots[(int64_t)i * kSpanWords + kSpanDeferItem];
+            if (item < (uint32_t)P.total_items) one((int)item);
+            __syncthreads();
+        }
     } else {
-        FusedBlock<R, false, 0, AUX> fb(P, lds);
-        run(fb);
+        one(xcd_contiguous_item(P.total_items));
     }
 }
-
 
 // =============================================================================================
 // Window and parameters apart from the block kernel (kWinApart): Adam direction from the window
@@ -2322,20 +2545,24 @@ static int launch_span_one(int pass, unsigned grid, int lds_bytes, hipStream_t s
     constexpr int kFirst =
         (R::kBF16 && R::kC <= kClass2 && AUX == 0) ? kWavesThreeWG : kMinWaves;
     // grid == 0: the preparation only, as in launch_fused_one
+#define MA_SPAN_CASE(PASS_, WAVES_, LDS_)                                                      \
+    case PASS_:                                                                                \
+        if (grid == 0) return allow_big_lds(span_step_kernel<R, WAVES_, PASS_, AUX>, LDS_);    \
+        return launch_kernel(span_step_kernel<R, WAVES_, PASS_, AUX>, dim3(grid), kWG, LDS_, s, P);
     switch (pass) {
-        case 1:
-            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 1, AUX>, lds_bytes);
-            return launch_kernel(span_step_kernel<R, kFirst, 1, AUX>, dim3(grid), kWG, lds_bytes, s, P);
-        case 2:
-            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 2, AUX>, lds_bytes);
-            return launch_kernel(span_step_kernel<R, kFirst, 2, AUX>, dim3(grid), kWG, lds_bytes, s, P);
-        case 4:
-            if (grid == 0) return allow_big_lds(span_step_kernel<R, kFirst, 4, AUX>, lds_bytes);
-            return launch_kernel(span_step_kernel<R, kFirst, 4, AUX>, dim3(grid), kWG, lds_bytes, s, P);
-        default:  // needs the kSh* words only
-            if (grid == 0) return 0;
-            return launch_kernel(span_step_kernel<R, kMinWaves, 3, AUX>, dim3(grid), kWG, kMiscBytes, s, P);
+        MA_SPAN_CASE(1, kFirst, lds_bytes)
+        MA_SPAN_CASE(2, kFirst, lds_bytes)
+        MA_SPAN_CASE(4, kFirst, lds_bytes)
+        MA_SPAN_CASE(3, kMinWaves, kMiscBytes)  // needs the kSh* words only
     }
+    if constexpr (AUX == 0) {  // the one-pass form and its sweeps
+        switch (pass) {
+            MA_SPAN_CASE(6, kFirst, lds_bytes)
+            MA_SPAN_CASE(8, kMinWaves, kMiscBytes)
+        }
+    }
+#undef MA_SPAN_CASE
+    return MA_ERR_ARG;
 }
 
 template <template <int> class RT, int AUX = 0>

@@ -4,6 +4,7 @@
 #include "ma_block.hpp"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -220,6 +221,15 @@ __global__ __launch_bounds__(kWG) void param_update_kernel(int64_t d, T *p, cons
         pv[e] = x + prod;
     }
     store8(p + i0, 0, n, vec, pv);
+}
+
+// Start state of the workspace of a call of the one-pass form: per block (two uint4) the four
+// extremes as all-ones words ("not published"), then zeros (flags, counts).
+__global__ __launch_bounds__(kWG) void span_clear_kernel(uint4 *ws, int64_t n16) {
+    for (int64_t i = (int64_t)blockIdx.x * kWG + threadIdx.x; i < n16; i += (int64_t)gridDim.x * kWG) {
+        const uint32_t w = (i & 1) ? 0u : 0xffffffffu;
+        ws[i] = make_uint4(w, w, w, w);
+    }
 }
 
 // ---- standalone top-k (+ gather + zero) ---------------------------------------------------------
@@ -494,6 +504,20 @@ static int fused_check(const ma_tensor *t, const ma_hyper *h, bool dense = false
 }
 
 constexpr int kSpanMaxBlocks = 64;  // top-k blocks one quantisation block may touch
+constexpr unsigned kSweepGroups = 256;  // workgroups of the sweep behind a one-pass launch
+
+// Polls a workgroup of the one-pass form spends at most on one neighbour's flag (each a sleep
+// of some 500 cycles and a load from device memory, say 2 us).  MA_SPAN_SPIN_LIMIT overrides
+// it: 0 makes every block give up at once and take the second pass, which is how the tests
+// reach that path.
+static int span_spin_limit() {
+    const char *e = getenv("MA_SPAN_SPIN_LIMIT");
+    if (e && *e) {
+        const long v = strtol(e, nullptr, 10);
+        return v < 0 ? 0 : v > 1000000 ? 1000000 : (int)v;
+    }
+    return 256;
+}
 
 // the two-pass route: 0 <= alpha < 1, quantisation blocks a multiple of 8 and at least as long
 // as the top-k blocks
@@ -515,7 +539,7 @@ static int span_check(const ma_tensor *t, const ma_hyper *h, double alpha) {
 
 static inline int64_t span_ws_bytes(const ma_tensor *t, const ma_hyper *h) {
     const Geometry g = geometry(t->d, h->d_block_size, h->k_init);
-    return (g.n_full + (g.tail > 0 ? 1 : 0)) * 16;  // 4 floats per block
+    return (g.n_full + (g.tail > 0 ? 1 : 0)) * kSpanWords * 4;
 }
 
 }  // namespace ma
@@ -535,7 +559,7 @@ const char *ma_error_string(int code) {
         case MA_ERR_LDS: return "launch would need more than 160 KB of LDS";
         case MA_ERR_WORKSPACE:
             return "list needs more workspace than ma_spanning_step_static holds "
-                   "(16 bytes per top-k block, MA_STATIC_WORKSPACE_BYTES in all)";
+                   "(32 bytes per top-k block, MA_STATIC_WORKSPACE_BYTES in all)";
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "unknown error";
@@ -768,10 +792,10 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
         }
     }
     if (n_tensors == 0) return 0;
+    int64_t ws_need = 0;
     if (span) {
-        int64_t need = 0;
-        for (int i = 0; i < n_tensors; ++i) need += span_ws_bytes(&tensors[i], h);
-        if (!ws || ws_bytes < need || ((uintptr_t)ws & 15) != 0) return MA_ERR_ARG;
+        for (int i = 0; i < n_tensors; ++i) ws_need += span_ws_bytes(&tensors[i], h);
+        if (!ws || ws_bytes < ws_need || ((uintptr_t)ws & 15) != 0) return MA_ERR_ARG;
     }
     hipStream_t s = (hipStream_t)stream;
     int q_shift = 0;
@@ -829,6 +853,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.keep = (float)(1.0 - alpha);
             P.metrics = (aux & kAuxLog) ? metrics + items_before * kMetricSlots : nullptr;
             P.win_apart = 0;
+            P.spin_limit = span_spin_limit();
             plan.back().kind = kWholeStep;
             int rc = P.L.total > kLdsLimit ? MA_ERR_LDS : 0;
             if (!span && !dense && !aux && P.L.cell_bytes == 0) {
@@ -895,8 +920,18 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
 
     // Two rounds over the plan: the first prepares every launch (kernel attributes: all that
     // can fail apart from a launch itself), the second launches.
+    // the one-pass form of the two-pass route (every step but a logging one) starts from a
+    // cleared workspace: its flags and counts are set as the blocks go
+    const bool one_pass = span && !aux && !(alpha > 0.0);
     for (int round = 0; round < 2; ++round)
     for (const PlannedLaunch &L : plan) {
+        if (one_pass && round == 1 && &L == &plan.front()) {
+            const int64_t n16 = ws_need / 16;
+            const unsigned cg = (unsigned)((n16 + kWG - 1) / kWG < 4096 ? (n16 + kWG - 1) / kWG : 4096);
+            const int rc0 = launch_kernel(span_clear_kernel, dim3(cg), kWG, 0, s,
+                                          reinterpret_cast<uint4 *>(ws), n16);
+            if (rc0) return rc0;
+        }
         const FusedParams &P = L.P;
         const unsigned grid = round == 0 ? 0u : (unsigned)P.total_items;
         const bool bf16 = h->dtype == MA_BF16;
@@ -920,14 +955,19 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             rc = bf16 ? launch_fused_bf16(L.C, grid, P.L.total, s, P)
                       : launch_fused_f32(L.C, grid, P.L.total, s, P);
         } else {
-            const int passes[2] = {alpha > 0.0 ? 1 : 4, alpha > 0.0 ? 2 : 3};
+            // alpha > 0 and logging steps: two passes; else one pass and the sweep over the
+            // blocks it deferred
+            const int passes[2] = {alpha > 0.0 ? 1 : one_pass ? 6 : 4,
+                                   alpha > 0.0 ? 2 : one_pass ? 8 : 3};
             for (int i = 0; i < 2 && rc == 0; ++i) {
+                unsigned g2 = grid;
+                if (one_pass && i == 1 && grid > kSweepGroups) g2 = kSweepGroups;
                 if (aux)
-                    rc = bf16 ? launch_span_log_bf16(L.C, passes[i], grid, P.L.total, s, P)
-                              : launch_span_log_f32(L.C, passes[i], grid, P.L.total, s, P);
+                    rc = bf16 ? launch_span_log_bf16(L.C, passes[i], g2, P.L.total, s, P)
+                              : launch_span_log_f32(L.C, passes[i], g2, P.L.total, s, P);
                 else
-                    rc = bf16 ? launch_span_bf16(L.C, passes[i], grid, P.L.total, s, P)
-                              : launch_span_f32(L.C, passes[i], grid, P.L.total, s, P);
+                    rc = bf16 ? launch_span_bf16(L.C, passes[i], g2, P.L.total, s, P)
+                              : launch_span_f32(L.C, passes[i], g2, P.L.total, s, P);
             }
         }
         // A launch the runtime refuses after an earlier one of the same call has started leaves

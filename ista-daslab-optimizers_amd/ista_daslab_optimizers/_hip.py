@@ -15,7 +15,7 @@ MA_ERR_ARG = -1
 MA_ERR_NOT_FUSABLE = -5
 MA_ERR_LDS = -6
 MA_ERR_WORKSPACE = -7
-MA_STATIC_WORKSPACE_BYTES = 8 << 20
+MA_STATIC_WORKSPACE_BYTES = 16 << 20
 MA_ROUTE_FUSED, MA_ROUTE_DENSIFIED, MA_ROUTE_SPANNING, MA_ROUTE_QUANT_ERR = 0, 1, 2, 3
 MA_MAX_WINDOW = 64
 

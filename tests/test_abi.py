@@ -136,7 +136,7 @@ def test_spanning_step_check_and_workspace():
     assert chk(0.5) == _hip.MA_ERR_NOT_FUSABLE
     h.quant_block_size = 100000
     arr = (_hip.MaTensor * 2)(t, t)
-    assert _hip.lib.ma_spanning_step_workspace(arr, 2, ctypes.byref(h)) == 2 * 3 * 16
+    assert _hip.lib.ma_spanning_step_workspace(arr, 2, ctypes.byref(h)) == 2 * 3 * 32
     # too small a workspace is refused before anything is launched
     rc = _hip.lib.ma_spanning_step(arr, 2, ctypes.byref(h), 0.5, 0x10000, 16, None)
     assert rc == -1  # MA_ERR_ARG

@@ -76,7 +76,8 @@ def test_static_scratch_step_equals_workspace_step(alpha):
         assert _call("workspace", want, opt, alpha, 4) == 0
         assert _call("static", got, opt, alpha, 4) == 0
         for i, (a, b) in zip(which, zip(got, want)):
-            for key in KEYS + ("p", "g"):
+            # (not the gradient buffer: the step may or may not leave the residual there)
+            for key in KEYS + ("p",):
                 assert torch.equal(a[key].view(torch.uint8).view(-1),
                                    b[key].view(torch.uint8).view(-1)), (alpha, which, i, key)
         # the step did something: parameters moved and codes were written
@@ -88,7 +89,7 @@ def test_static_scratch_step_equals_workspace_step(alpha):
 def test_static_scratch_step_rejects_lists_beyond_its_array():
     """More top-k blocks than the array has room for: refused before anything is launched."""
     from ista_daslab_optimizers import _hip
-    n_blocks = _hip.MA_STATIC_WORKSPACE_BYTES // 16 + 1
+    n_blocks = _hip.MA_STATIC_WORKSPACE_BYTES // 32 + 1
     t = (_hip.MaTensor * 1)()
     for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
         setattr(t[0], f, 0x10000)
