@@ -168,7 +168,7 @@ int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
 int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
 
 /* ma_fused_step for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), same
- * conditions but quant_block_size at most 512, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and
+ * conditions, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and
  * statistics; window -> Adam direction, + alpha * Qinv(e1); p update; the error feedback that is
  * stored is Q((1 - alpha) * Qinv(e1)) with statistics of its own. */
 int ma_fused_step_densified(const ma_tensor *tensors /* host */, int n_tensors,

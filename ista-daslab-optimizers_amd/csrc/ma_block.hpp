@@ -1271,6 +1271,31 @@ struct FusedBlock {
         uint8_t *err = G.D.err + (G.e0 >> 1);
         uint16_t *mnp = G.D.mn + (G.e0 >> q_shift);
         uint16_t *mxp = G.D.mx + (G.e0 >> q_shift);
+        // quantisation blocks of 1024 to 4096 elements: the extremes of the 512-element
+        // stretches meet in LDS, as in quantize
+        const bool long_q = QL == 0 && ql > kWave;
+        float *stretch = reinterpret_cast<float *>(hist);  // [wave * C + chunk][min, max]
+        if (long_q) {
+            __syncthreads();  // the selection may still be reading its lists there
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const int off = chunk_off<C>(wave, c, lane);
+                float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) {
+                    if (FULL || off + e < n) {
+                        mn = fmin_raw(mn, r.val(c, e));
+                        mx = fmax_raw(mx, r.val(c, e));
+                    }
+                }
+                group_minmax<0>(mn, mx, kWave);
+                if (lane == 0) {
+                    stretch[(wave * C + c) * 2] = mn;
+                    stretch[(wave * C + c) * 2 + 1] = mx;
+                }
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int off = chunk_off<C>(wave, c, lane);
@@ -1289,15 +1314,26 @@ struct FusedBlock {
                     }
                 }
             }
-            group_minmax<QL>(mn, mx, ql);
+            if (long_q) {
+                const int per = ql / kWave;  // stretches per quantisation block
+                const int first = (wave * C + c) / per * per;
+                mn = INFINITY;
+                mx = -INFINITY;
+                for (int j = 0; j < per; ++j) {
+                    mn = fmin_raw(mn, stretch[(first + j) * 2]);
+                    mx = fmax_raw(mx, stretch[(first + j) * 2 + 1]);
+                }
+            } else {
+                group_minmax<QL>(mn, mx, ql);
+            }
             const uint32_t mnb = f2bf(mn), mxb = f2bf(mx);
             dstat[c] = mnb | mxb << 16;
             dcodes[c] = 0;
             float r2[8];
             float mn2 = INFINITY, mx2 = -INFINITY;
+            const float mnf = bf2f(mnb);
+            const float u = div15(bf2f(mxb) - mnf, d15);
             if (FULL || off < n) {
-                const float mnf = bf2f(mnb);
-                const float u = div15(bf2f(mxb) - mnf, d15);
                 float cf[8];
                 codes8(x, mnf, u, cf);
 #pragma unroll
@@ -1316,7 +1352,24 @@ struct FusedBlock {
                     }
                 }
             }
-            group_minmax<QL>(mn2, mx2, ql);
+            if (long_q) {
+                // r2 does not decrease with the code, nor the code with the element: the
+                // extremes of r2 over the quantisation block are r2 at the codes of the
+                // extremes of r, which every chunk of the block knows
+                float ext[8], ce[8];
+#pragma unroll
+                for (int e = 0; e < kChunk; ++e) ext[e] = (e & 1) ? mx : mn;
+                codes8(ext, mnf, u, ce);
+                float lo = ce[0] * u, hi = ce[1] * u;
+                lo = lo + mnf;
+                hi = hi + mnf;
+                lo = P.keep * lo;
+                hi = P.keep * hi;
+                mn2 = to_elem(0.0f + lo);
+                mx2 = to_elem(0.0f + hi);
+            } else {
+                group_minmax<QL>(mn2, mx2, ql);
+            }
             const uint32_t mn2b = f2bf(mn2), mx2b = f2bf(mx2);
             if (FULL || off < n) {
                 if ((lane & (ql - 1)) == 0) {

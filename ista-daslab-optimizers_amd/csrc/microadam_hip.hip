@@ -485,13 +485,14 @@ static int common_check(const ma_tensor *t, const ma_hyper *h, Geometry *g) {
     return 0;
 }
 
-// dense: with 0 < alpha < 1 (whose two quantisations stay inside a wave's stretch of 512)
+// dense: with 0 < alpha < 1
 static int fused_check(const ma_tensor *t, const ma_hyper *h, bool dense = false) {
     Geometry g;
     const int rc = common_check(t, h, &g);
     if (rc) return rc;
     const int64_t q = h->quant_block_size;
-    if (q < 8 || q > (dense ? 512 : 4096) || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
+    (void)dense;
+    if (q < 8 || q > 4096 || (q & (q - 1)) != 0) return MA_ERR_NOT_FUSABLE;
     if (t->d < q) return MA_ERR_NOT_FUSABLE;
     const bool single = t->d <= h->d_block_size;
     if (!single && (g.dbs % q != 0 || g.dbs % 8 != 0)) return MA_ERR_NOT_FUSABLE;

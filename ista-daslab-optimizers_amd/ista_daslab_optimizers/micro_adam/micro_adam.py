@@ -228,8 +228,7 @@ class MicroAdam(torch.optim.Optimizer):
                 return FUSED_QUANT_ERR
             if self.alpha == 0:
                 return FUSED
-            if self.quant_block_size <= 512:  # (ma_fused_step_densified's own limit)
-                return FUSED_DENSIFIED
+            return FUSED_DENSIFIED
         if self.alpha == -2:
             return OP_BY_OP
         if _hip.lib.ma_spanning_step_check(ctypes.byref(probe), ctypes.byref(h),

@@ -97,8 +97,6 @@ GENERAL_CASES = [
     ([999], torch.float32, 2, 100, 0.03, 0.25, 0.01, 400, 5),
     ([20480 * 3 + 77], torch.bfloat16, 4, 100001, 0.01, 0.5, 0.0, 20480, 6),
     ([50, 20], torch.bfloat16, 3, 60, 0.1, 0.0, 0.0, 20480, 4),
-    # 0 < alpha < 1 with quantisation blocks between 512 elements and the top-k block
-    ([20480 * 2 + 4096], torch.bfloat16, 3, 1024, 0.01, 0.5, 0.0, 20480, 4),
     # alpha == -2 with quantisation blocks that the one-pass kernels do not take
     ([4100, 33], torch.bfloat16, 3, 1000, 0.01, -2, 0.0, 1024, 5),
 ]
@@ -158,6 +156,10 @@ FUSED_DENSIFIED_CASES = [
     ([5000], torch.float32, 3, 64, 0.02, 0.7, 0.0, 2048, 7),
     ([20480 + 4096], torch.float32, 10, 32, 0.01, 0.1, 0.01, 20480, 12),
     ([1001, 777], torch.bfloat16, 3, 64, 0.03, 0.5, 0.0, 20480, 5),   # odd d: partial chunks
+    # quantisation blocks longer than the 512 elements a wave holds per chunk
+    ([20480 * 2 + 4096, 3000], torch.bfloat16, 3, 1024, 0.01, 0.5, 0.0, 20480, 4),
+    ([20480 + 5000], torch.float32, 4, 4096, 0.01, 0.3, 0.01, 20480, 6),
+    ([32768 + 9000], torch.bfloat16, 3, 2048, 0.01, 0.7, 0.0, 32768, 5),
 ]
 
 
