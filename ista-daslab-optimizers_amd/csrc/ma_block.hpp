@@ -2184,15 +2184,13 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             // (the parameters are asked for once the residual has left the registers: both
             // held through the wait and the codes would not fit the register budget of three
             // workgroups per CU)
-            fb.wide = fb.wide_window(G);
-            if (fb.wide) fb.load_window_wide(G); else fb.load_window(G);
             if (fb.template span_await<false>(G, S)) {
                 fb.template span_codes_stage<true>(G, S);
             } else {
                 fb.span_defer(G);
                 list_deferred(item);
             }
-            fb.load_params(G);
+            fb.load_params_window(G);
             fb.update(G);
         }
         constexpr unsigned kUnused = 1u << kMtQuantErr | 1u << kMtQuantErrZeros | 3u << 6;
