@@ -108,6 +108,13 @@ def error_string(code):
 
 
 def check(code, what):
+    """Negative codes reject the call before anything was launched.  A positive code is the
+    hipError_t of a launch the runtime refused: launches before it have run, so a step call may
+    be part-way applied and must not be repeated."""
+    if code > 0:
+        raise RuntimeError(f"{what}: the HIP runtime refused a launch: {error_string(code)} "
+                           f"(hipError_t {code}); earlier launches of the call have run, so "
+                           "restore the optimizer from a checkpoint instead of stepping again")
     if code != 0:
         raise RuntimeError(f"{what} failed: {error_string(code)} (code {code})")
 
