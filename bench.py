@@ -319,11 +319,13 @@ def calibration(args):
                            e.data_ptr(), sink.data_ptr(), _hip.stream_ptr())
         return run
 
-    moved = {0: nbytes, 1: nbytes, 2: 2 * nbytes, 3: 3 * nbytes, 4: 3 * nbytes + nbytes // 2}
+    moved = {0: nbytes, 1: nbytes, 2: 2 * nbytes, 3: 3 * nbytes, 4: 3 * nbytes + nbytes // 2,
+             5: 2 * nbytes}
     names = {0: "read", 1: "write", 2: "copy", 3: "update (2 reads : 1 write)",
-             4: "step streams (g, p, EF read; p, EF written)"}
+             4: "step streams (g, p, EF read; p, EF written)",
+             5: "write, then read the same 40 KiB back"}
     rows = []
-    for mode in range(5):
+    for mode in range(6):
         for nt in (1, 0):
             for wgs in (0, 256 * 3 * 4):
                 ms = timed(probe(mode, nt, wgs))

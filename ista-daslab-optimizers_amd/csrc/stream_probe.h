@@ -18,6 +18,8 @@ extern "C" {
  * mode 0: reads a.  1: writes c.  2: c = a.  3: b = a + b (two reads, one write).
  * 4: reads a, b and e, writes b and e, with e a quarter as long as a (the step's gradient,
  *    parameter and 4-bit error-feedback streams: 7 bytes per bf16 element).
+ * 5: writes c and reads the same stretch back once the stores have completed (does the L2 serve
+ *    lines that were just written?).
  * nontemporal != 0 uses the cache-bypassing loads and stores the step uses.  workgroups > 0
  * caps the grid (each workgroup then takes several stretches in turn), 0 launches one per
  * stretch.  sink: 4 bytes of device memory (keeps the read-only mode's loads alive).  Used by

@@ -31,6 +31,9 @@ __device__ __forceinline__ void st(u4 *p, u4 v) {
 
 // MODE 0: read a.  1: write c.  2: c = a.  3: b = f(a, b) (two reads, one write: the step's mix).
 // 4: the step's three large streams: reads a (2 B per element), b (2 B), e (0.5 B); writes b, e.
+// 5: writes c and, once the stores have completed and this CU's L1 is emptied, reads the same
+//    stretch back: what the L2 fetches for it tells whether lines just written are served from
+//    the L2 (a workgroup handing data to another of its XCD would rely on that).
 template <int MODE, bool NT>
 __global__ __launch_bounds__(kThreads) void stream_kernel(const u4 *a, u4 *b, u4 *c, uint32_t *e,
                                                           int64_t segments, uint32_t *sink) {
@@ -58,9 +61,18 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(const u4 *a, u4 *b, u4
                 st<NT>(b + i, va[k] + vb[k] + ve[k]);
                 e[i] = ve[k] ^ va[k].x;
             }
+            if (MODE == 5) st<NT>(c + i, u4{(uint32_t)i, 1u, 2u, 3u});
+        }
+        if (MODE == 5) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            asm volatile("buffer_inv sc0" ::: "memory");
+#pragma unroll
+            for (int k = 0; k < kChunks; ++k)
+                acc ^= ld<false>(c + base + (wave * kChunks + k) * 64 + lane);
         }
     }
-    if (MODE == 0 && (acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) *sink = acc.x;
+    if ((MODE == 0 || MODE == 5) && (acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) *sink = acc.x;
 }
 
 template <int MODE>
@@ -86,7 +98,7 @@ extern "C" int ma_stream_probe(int mode, int nontemporal, int64_t bytes, int64_t
     const int64_t segments = bytes / kSegBytes;
     if (segments > 0x7fffffff) return kProbeErrArg;
     const bool need_a = mode == 0 || mode == 2 || mode == 3 || mode == 4;
-    const bool need_b = mode == 3 || mode == 4, need_c = mode == 1 || mode == 2;
+    const bool need_b = mode == 3 || mode == 4, need_c = mode == 1 || mode == 2 || mode == 5;
     if ((need_a && !a) || (need_b && !b) || (need_c && !c) || (mode == 4 && !e)) return kProbeErrArg;
     const unsigned grid = (unsigned)(workgroups > 0 && workgroups < segments ? workgroups : segments);
     hipStream_t s = (hipStream_t)stream;
@@ -96,6 +108,7 @@ extern "C" int ma_stream_probe(int mode, int nontemporal, int64_t bytes, int64_t
         case 2: return launch<2>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
         case 3: return launch<3>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
         case 4: return launch<4>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
+        case 5: return launch<5>(nontemporal != 0, grid, s, a, b, c, e, segments, sink);
     }
     return kProbeErrArg;
 }
