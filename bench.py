@@ -283,6 +283,44 @@ def bench_sparse_window(args):
     print(json.dumps(res))
 
 
+class LaunchEvents:
+    """Events on the launch stream right before and after every call of a step entry point of
+    the library (each call enqueues all launches of its tensors and returns): the device time of
+    a step is the time between them, added over the step's calls.  Events around step() as a
+    whole also count the host's work of a step whenever the stream is empty, which is the case
+    for the first steps after the synchronisation that starts the timed region."""
+    ENTRY_POINTS = ("ma_fused_step", "ma_fused_step_densified", "ma_fused_step_quant_err",
+                    "ma_spanning_step", "ma_logged_step")
+
+    def __init__(self):
+        import torch
+        from ista_daslab_optimizers import _hip
+        self.lib, self.steps, self.saved = _hip.lib, [], {}
+        for name in self.ENTRY_POINTS:
+            fn = getattr(self.lib, name)
+            self.saved[name] = fn
+
+            def timed(*a, _fn=fn):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                rc = _fn(*a)
+                e1.record()
+                self.steps[-1].append((e0, e1))
+                return rc
+            setattr(self.lib, name, timed)
+
+    def begin_step(self):
+        self.steps.append([])
+
+    def restore(self):
+        for name, fn in self.saved.items():
+            setattr(self.lib, name, fn)
+
+    def per_step_ms(self):
+        return [sum(a.elapsed_time(b) for a, b in step) for step in self.steps]
+
+
 def calibration(args):
     """Known-size streaming kernels on this device: the rate it sustains for reads, writes, a
     copy, the step's 2:1 read:write mix and the step's three large streams, with the step's own
@@ -453,18 +491,25 @@ def main():
         del src, dst
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
+    calls = LaunchEvents()
     host = 0.0  # time the host spends inside step() (the kernels run behind it)
     t0 = time.perf_counter()
     for i in range(args.steps):
         prepare(args.warmup + i)  # (its kernels run between the events of two steps)
         ev[i][0].record()
         h0 = time.perf_counter()
+        calls.begin_step()
         one_step(args.warmup + i)
         host += time.perf_counter() - h0
         ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    dev_series = [a.elapsed_time(b) for a, b in ev]  # in step order
+    calls.restore()
+    span_series = [a.elapsed_time(b) for a, b in ev]  # in step order
+    # the launches of a step, timed on their stream; the op-by-op route (one library call and a
+    # few torch kernels per operation) has no step entry point to bracket: its steps are
+    # timed from the events around step()
+    dev_series = calls.per_step_ms() if all(calls.steps) else span_series
     dev_ms = sorted(dev_series)
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = sum(dev_ms) / len(dev_ms)
@@ -506,7 +551,10 @@ def main():
                      "per": "step", "algorithmic_bytes": bpp * n_params,
                      "bytes_per_param": bpp, "device_ms_per_step": kernel_ms,
                      "device_ms_min": dev_ms[0], "device_ms_median": dev_ms[len(dev_ms) // 2],
-                     "device_ms_series": [round(x, 3) for x in dev_series]},
+                     "device_ms_series": [round(x, 3) for x in dev_series],
+                     # events around the whole of step(): on top of the launches, the host's
+                     # share of a step whenever the stream has run dry (the first timed steps)
+                     "step_events_ms_per_step": sum(span_series) / len(span_series)},
     }
     if not args.no_cpu_baseline:
         del grad_sets

@@ -74,6 +74,7 @@ struct FusedParams {
     int32_t d_block_size;
     int32_t q_shift;  // log2(quant_block_size)
     int32_t total_items;  // work items (blocks) of the launch
+    int32_t short_items;  // of them, at the end: tensors shorter than a top-k block, one item each
     // two-pass route (quantisation blocks at least as long as the top-k blocks)
     int32_t q_span;   // quantisation block length, a multiple of 8
     float alpha;      // share of the dequantised error feedback added to the update
@@ -2056,12 +2057,21 @@ struct FusedBlock {
 // chip's 8 XCDs in turn (workgroup i runs on XCD i % 8, each with its own L2); the items are
 // dealt out so that every XCD walks one contiguous eighth of the launch's blocks, which the
 // memory system serves measurably faster than eight interleaved walks (stores most of all).
-__device__ __forceinline__ int xcd_contiguous_item(int total_items) {
+// The launch's last `short_items` items (tensors shorter than a block, which finish early) are
+// dealt out apart, an eighth to every XCD behind its share of the others: the workgroups that
+// start last are then short ones, and the launch does not end on a round of full blocks.
+__device__ __forceinline__ int xcd_contiguous_item(int total_items, int short_items) {
     constexpr int kXcds = 8;
     const int bid = (int)blockIdx.x;
     const int x = bid % kXcds, j = bid / kXcds;
     const int q = total_items / kXcds, r = total_items % kXcds;
-    return x * q + (x < r ? x : r) + j;
+    const int qs = short_items / kXcds, rs = short_items % kXcds;
+    // XCD x runs all_here workgroups; items before its own, of either kind
+    const int all_here = q + (x < r ? 1 : 0), short_here = qs + (x < rs ? 1 : 0);
+    const int all_before = x * q + (x < r ? x : r), short_before = x * qs + (x < rs ? x : rs);
+    const int long_here = all_here - short_here, long_before = all_before - short_before;
+    return j < long_here ? long_before + j
+                         : (total_items - short_items) + short_before + (j - long_here);
 }
 
 // which tensor owns workgroup / work item `w` of the launch (first_block is ascending)
@@ -2085,7 +2095,7 @@ constexpr int kWinFused = 0, kWinApart = 2;
 template <class R, int MIN_WAVES, int QL, bool DENSE = false, int WIN = kWinFused, int AUX = 0>
 __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams P) {
     extern __shared__ __align__(16) unsigned char lds[];
-    const int item = xcd_contiguous_item(P.total_items);
+    const int item = xcd_contiguous_item(P.total_items, P.short_items);
     const int ti = find_tensor(P, item);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
     auto run = [&](auto &fb) {
@@ -2220,7 +2230,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
             __syncthreads();
         }
     } else {
-        one(xcd_contiguous_item(P.total_items));
+        one(xcd_contiguous_item(P.total_items, P.short_items));
     }
 }
 
@@ -2270,7 +2280,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
     uint32_t *sh = reinterpret_cast<uint32_t *>(lds);
     int *table = reinterpret_cast<int *>(lds + P.L.off_slot);
     float *sums = reinterpret_cast<float *>(lds + P.L.off_union);
-    const int item = xcd_contiguous_item(P.total_items);
+    const int item = xcd_contiguous_item(P.total_items, P.short_items);
     const int ti = find_tensor(P, item);
     const BlockGeo G = make_geo(P, ti, P.t[ti].blk0 + (item - P.t[ti].first_block));
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

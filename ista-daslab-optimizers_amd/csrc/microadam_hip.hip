@@ -828,17 +828,28 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     //      either steps every tensor or none
     std::vector<PlannedLaunch> plan;
     int64_t items_before = 0;  // work items of the launches laid out so far
+    // the two-pass route's workspace is handed out in the order the tensors are laid out, so the
+    // slots of a launch's tensors follow each other from those of its first tensor
+    int64_t ws_off = 0;
+    std::vector<int> order;
     for (int ci = 0; ci < 4; ++ci) {
-        int in_class = 0;
-        for (int i = 0; i < n_tensors; ++i)
-            if (cls[i] == ci) ++in_class;
+        // the class's tensors in list order, those shorter than a top-k block (one partial
+        // block each: they finish early) behind the others
+        order.clear();
+        for (int pass = 0; pass < 2; ++pass)
+            for (int i = 0; i < n_tensors; ++i) {
+                if (cls[i] != ci) continue;
+                const bool is_short = tensors[i].d < h->d_block_size;
+                if (is_short == (pass == 1)) order.push_back(i);
+            }
+        const int in_class = (int)order.size();
         if (in_class == 0) continue;
         // the class's tensors are spread evenly over as few launches as hold them (the
         // descriptors travel by value, kTensorsPerLaunch at most)
         const int launches = (in_class + kTensorsPerLaunch - 1) / kTensorsPerLaunch;
         const int per_launch = (in_class + launches - 1) / launches;
-        int count = 0;
-        int64_t items = 0, ws_off = 0;
+        int count = 0, short_items = 0;
+        int64_t items = 0;
         int dbs_max = 0, kb_max = 0;
         auto close = [&]() -> int {
             if (count == 0) return 0;
@@ -849,6 +860,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             P.d_block_size = d_block_size;
             P.q_shift = q_shift;
             P.total_items = (int32_t)items;
+            P.short_items = short_items;
             P.q_span = span ? (int32_t)h->quant_block_size : 0;
             P.alpha = (float)alpha;
             P.keep = (float)(1.0 - alpha);
@@ -870,17 +882,16 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                 plan.push_back(second);
             }
             items_before += items;
-            count = 0;
+            count = short_items = 0;
             items = 0;
             dbs_max = kb_max = 0;
             return rc;
         };
-        for (int i = 0; i < n_tensors; ++i) {
+        for (const int i : order) {
             const ma_tensor &t = tensors[i];
             const Geometry g = geometry(t.d, h->d_block_size, h->k_init);
             const int64_t ws_here = ws_off;
             if (span) ws_off += span_ws_bytes(&t, h);
-            if (cls[i] != ci) continue;
             const int64_t nb = g.n_full + (g.tail > 0 ? 1 : 0);
             if (count == per_launch || items + nb > 0x7fffffff) {
                 const int rc = close();
@@ -911,6 +922,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             D.ws = span ? reinterpret_cast<float *>(static_cast<char *>(ws) + ws_here)
                         : (aux & kAuxQuantErr) ? static_cast<float *>(t.quant_err) : nullptr;
             items += nb;
+            if (t.d < h->d_block_size) ++short_items;  // (nb == 1, and only short ones follow)
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;
             if (g.k_many > kb_max) kb_max = (int)g.k_many;
             ++count;
