@@ -141,6 +141,8 @@ typedef struct ma_tensor {
     void *quant_err;    /* st['quant_err'], `dtype`, d elements, MA:67-68; written by
                            ma_fused_step_quant_err (and ma_logged_step on that route), 16-byte
                            aligned; the other entry points ignore it (may be NULL) */
+    uint16_t *row_cuts; /* optional cache kept by ma_fused_step, no counterpart in the reference:
+                           m x ma_fused_step_row_cuts() words, or NULL; see there */
 } ma_tensor;
 
 typedef struct ma_hyper {
@@ -166,6 +168,22 @@ int ma_fused_step(const ma_tensor *tensors /* host */, int n_tensors,
 /* 0 if ma_fused_step would accept this tensor under `hyper`, else the MA_ERR_* it would
  * return.  Host-only check, launches nothing. */
 int ma_fused_step_check(const ma_tensor *tensor /* host */, const ma_hyper *hyper /* host */);
+
+/* ma_fused_step steps tensors whose window has about as many entries as the tensor has
+ * coordinates (more than 2560 entries per top-k block, or more than 16 rows) in two launches; the
+ * second walks every window row in stretches of 512 coordinates and must know where each row
+ * crosses those boundaries.  With tensor->row_cuts == NULL it finds out by reading all rows at
+ * every step.  With a buffer of m x (this function's value) uint16 words, set to 0xffff before
+ * its first use and from then on written by nobody else, the first launch files the cuts of
+ * the row it writes and the second reads them: row r, block b, cut c (the number of entries of
+ * that block's stretch of row r whose coordinate is below 512 c) is word
+ * (r * blocks + b) * cuts_per_block + c, cuts_per_block = ceil(min(d, d_block_size) / 512) + 1.
+ * A row whose first cut is 0xffff is taken as unknown and read in full.  Whoever else rewrites a
+ * window row of the tensor (another entry point, a loaded checkpoint) must set that row's
+ * words to 0xffff again.  Returns the words per row, 0 if the tensor's step would not use them,
+ * negative MA_ERR_* for bad arguments. */
+int64_t ma_fused_step_row_cuts(const ma_tensor *tensor, const ma_hyper *hyper);
+
 
 /* ma_fused_step for 0 < alpha < 1 (densify_update_using_ef, MA:296-298 and MA:311-316), same
  * conditions, still one pass per top-k block: e1 = Q(residual) stays in registers as codes and

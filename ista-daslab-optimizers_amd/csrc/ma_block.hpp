@@ -59,7 +59,9 @@ struct TensorDesc {
     int32_t apply_decay;
     int32_t blk0;         // block of the tensor that its first work item stands for
     float *ws;            // two-pass route: per-block extremes of the residual;
-                          // alpha == -2: st['quant_err'] (elements of the data's type); else unused
+                          // alpha == -2: st['quant_err'] (elements of the data's type);
+                          // two-launch form of dense windows: the cache of row cuts (uint16
+                          // words) or null; else unused
 };
 // The descriptors travel by value in the kernel arguments (112 bytes each; the runtime passes
 // arguments of this size intact).  Fewer, longer launches: each launch ends with a partly
@@ -102,6 +104,21 @@ struct FusedParams {
 //            the parameter's type) before the Adam step.
 constexpr int kAuxLog = 1, kAuxQuantErr = 2;
 constexpr int kSpanWords = 8;  // workspace words per top-k block of the two-pass route
+constexpr int kRowCutStep = 512;  // coordinates between two cuts of a window row
+
+// Layout of a tensor's cache of row cuts: (row, block, cut) -> word
+struct RowCuts {
+    int64_t blocks;
+    int per_block;
+    __host__ __device__ RowCuts(int64_t d, int64_t d_block_size) {
+        const int64_t dbs = d < d_block_size ? d : d_block_size;
+        blocks = (d + dbs - 1) / dbs;
+        per_block = (int)((dbs + kRowCutStep - 1) / kRowCutStep) + 1;
+    }
+    __host__ __device__ int64_t at(int64_t row, int64_t block) const {
+        return (row * blocks + block) * per_block;
+    }
+};
 constexpr int kMetricSlots = 8;
 enum { kMtQuantErr = 0, kMtGrad = 1, kMtUpdate = 2, kMtError = 3, kMtUpdateZeros = 4, kMtQuantErrZeros = 5 };
 
@@ -489,6 +506,7 @@ struct FusedBlock {
                 slot_clear = topk_done && P.L.slot_cells == C * kRound;
             }
         }
+        row_sorted = !topk_done;  // the general selection lists its entries by coordinate
         if (!topk_done) {
             uint32_t T;
             int take_eq;
@@ -502,6 +520,32 @@ struct FusedBlock {
         for (int j = tid; j < kb; j += kWG) {
             Irow[(unsigned)j] = (int16_t)sel_idx[j];
             Vrow[(unsigned)j] = sel_val[j];
+        }
+    }
+
+    // Two-launch form: where the row just written (still in sel_idx) crosses the multiples of
+    // kRowCutStep coordinates goes to the tensor's cache of row cuts, if it keeps one, for
+    // window_param_kernel: cut c = number of entries with coordinate < c * kRowCutStep.  A row
+    // that is not listed by coordinate is marked unknown.
+    bool row_sorted;
+    __device__ __forceinline__ void file_row_cuts(const BlockGeo &G) {
+        uint16_t *cuts = reinterpret_cast<uint16_t *>(G.D.ws);
+        if (cuts == nullptr) return;
+        const RowCuts where(G.D.d, P.d_block_size);
+        uint16_t *mine = cuts + where.at(G.D.row, block_id(G));
+        const int nch = (G.n + kRowCutStep - 1) / kRowCutStep;
+        if (!row_sorted) {
+            if (tid == 0) mine[0] = 0xffffu;
+            return;
+        }
+        if (tid <= nch) {
+            const int bound = tid * kRowCutStep;
+            int lo = 0, hi = G.kb;  // first entry whose coordinate is not below `bound`
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if ((int)sel_idx[mid] < bound) lo = mid + 1; else hi = mid;
+            }
+            mine[tid] = (uint16_t)lo;
         }
     }
 
@@ -2102,6 +2146,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void fused_step_kernel(FusedParams 
         fb.load_grad_inputs(G);
         fb.dequant(G);
         fb.topk_and_row(G);
+        if constexpr (WIN == kWinApart) fb.file_row_cuts(G);
         if constexpr (DENSE) {
             fb.quantize_dense(G);
             fb.load_params(G);
@@ -2259,6 +2304,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void span_step_kernel(FusedParams P
 // =============================================================================================
 constexpr int kWinShift = 9;
 constexpr int kWinChunk = 1 << kWinShift;  // coordinates per chunk: 8 for each of 64 lanes
+static_assert(kWinChunk == kRowCutStep, "the cached row cuts are the chunk boundaries");
 constexpr int kWinRowBatch = 10;    // rows whose stretches are requested together
 
 // two window entries as they lie in memory, from any 2-byte boundary (the hardware takes
@@ -2298,9 +2344,31 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
     //      Thread t takes the entries 2t and 2t + 1 of every row (one load), the entry before
     //      them comes from the lane below, for lane 0 from memory.
     if (tid == 0) sh[0] = 0;
+    __syncthreads();
+    // from the tensor's cache of row cuts, when it keeps one and knows every live row
+    // (fused_step_kernel files a row's cuts when it writes the row in coordinate order)
+    const uint16_t *cuts = reinterpret_cast<const uint16_t *>(G.D.ws);
+    bool cached = cuts != nullptr;
+    if (cached) {
+        const RowCuts where(G.D.d, P.d_block_size);
+        const int64_t block = G.e0 / (G.D.d < P.d_block_size ? G.D.d : P.d_block_size);
+        bool unknown = false;
+        for (int i = tid; i < rows * stride; i += kWG) {
+            const int r = i / stride, ch = i - r * stride;
+            const uint32_t cut = cuts[where.at(r, block) + ch];
+            table[i] = 2 * (int)cut;
+            if (ch == 0 && cut != 0) unknown = true;
+        }
+        if (unknown) atomicOr(&sh[0], 2u);
+        __syncthreads();
+        cached = sh[0] == 0;
+        __syncthreads();
+        if (tid == 0) sh[0] = 0;
+    }
+    bool bad = false;
+    if (!cached) {
     for (int i = tid; i < rows * stride; i += kWG) table[i] = 2 * kb;
     __syncthreads();
-    bool bad = false;
     for (int j0 = 0; j0 < kb; j0 += 2 * kWG) {
         const int j = j0 + 2 * tid;
         for (int r0 = 0; r0 < rows; r0 += kWinRowBatch) {
@@ -2345,6 +2413,7 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
                 }
             }
         }
+    }
     }
     if (bad) atomicOr(&sh[0], 1u);
     __syncthreads();

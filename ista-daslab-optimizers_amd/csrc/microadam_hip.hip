@@ -729,6 +729,32 @@ int ma_fused_step_check(const ma_tensor *tensor, const ma_hyper *hyper) {
     return fused_check(tensor, hyper);
 }
 
+// Does ma_fused_step (alpha == 0, no logging) step a tensor of d elements in two launches?  Its
+// window does not fit the one-pass stage of the block kernel then.
+static bool window_apart(int64_t d, const ma_hyper *h, int elem_bytes) {
+    const Geometry g = geometry(d, h->d_block_size, h->k_init);
+    return plan_lds((int)g.dbs, (int)g.k_many, h->m, elem_bytes, true, true).cell_bytes == 0;
+}
+
+// words per window row of the cache of chunk cuts, see the header
+static int64_t row_cut_words(int64_t d, const ma_hyper *h) {
+    const Geometry g = geometry(d, h->d_block_size, h->k_init);
+    const int64_t blocks = g.n_full + (g.tail > 0 ? 1 : 0);
+    return blocks * ((g.dbs + kWinChunk - 1) / kWinChunk + 1);
+}
+
+int64_t ma_fused_step_row_cuts(const ma_tensor *tensor, const ma_hyper *hyper) {
+    if (!tensor || !hyper) return MA_ERR_ARG;
+    const int rc = fused_check(tensor, hyper);
+    if (rc) return rc;
+    const Geometry g = geometry(tensor->d, hyper->d_block_size, hyper->k_init);
+    // only rows of more than 512 entries per block are written in coordinate order, which is
+    // what the cuts describe
+    if (!window_apart(tensor->d, hyper, hyper->dtype == MA_BF16 ? 2 : 4) || g.k_many <= kWG)
+        return 0;
+    return row_cut_words(tensor->d, hyper);
+}
+
 // One planned launch of a step: the kernel's parameters and the register-tile class it runs in.
 struct PlannedLaunch {
     FusedParams P;
@@ -831,14 +857,22 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
     // the two-pass route's workspace is handed out in the order the tensors are laid out, so the
     // slots of a launch's tensors follow each other from those of its first tensor
     int64_t ws_off = 0;
+    // tensors whose window is too large for the one-pass stage are stepped in two launches
+    // (block part, window part) of their own, whatever else the call holds: which form a tensor
+    // takes depends on its sizes alone
+    std::vector<char> apart(n_tensors, 0);
+    if (!span && !dense && !aux)
+        for (int i = 0; i < n_tensors; ++i)
+            apart[i] = window_apart(tensors[i].d, h, elem_bytes) ? 1 : 0;
     std::vector<int> order;
-    for (int ci = 0; ci < 4; ++ci) {
-        // the class's tensors in list order, those shorter than a top-k block (one partial
-        // block each: they finish early) behind the others
+    for (int ci = 0; ci < 4; ++ci)
+    for (int form = 0; form < 2; ++form) {
+        // the class's tensors of this form in list order, those shorter than a top-k block (one
+        // partial block each: they finish early) behind the others
         order.clear();
         for (int pass = 0; pass < 2; ++pass)
             for (int i = 0; i < n_tensors; ++i) {
-                if (cls[i] != ci) continue;
+                if (cls[i] != ci || apart[i] != form) continue;
                 const bool is_short = tensors[i].d < h->d_block_size;
                 if (is_short == (pass == 1)) order.push_back(i);
             }
@@ -920,7 +954,9 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
             D.decay = (float)(1.0 - t.lr * t.weight_decay);
             D.blk0 = 0;
             D.ws = span ? reinterpret_cast<float *>(static_cast<char *>(ws) + ws_here)
-                        : (aux & kAuxQuantErr) ? static_cast<float *>(t.quant_err) : nullptr;
+                   : (aux & kAuxQuantErr) ? static_cast<float *>(t.quant_err)
+                   : apart[i] ? reinterpret_cast<float *>(t.row_cuts)
+                              : nullptr;
             items += nb;
             if (t.d < h->d_block_size) ++short_items;  // (nb == 1, and only short ones follow)
             if (g.dbs > dbs_max) dbs_max = (int)g.dbs;

@@ -27,7 +27,7 @@ class MaTensor(ctypes.Structure):
                 ("I", ctypes.c_void_p), ("V", ctypes.c_void_p), ("d", ctypes.c_int64),
                 ("k", ctypes.c_int64), ("lr", ctypes.c_double), ("weight_decay", ctypes.c_double),
                 ("index", ctypes.c_int32), ("reserved", ctypes.c_int32),
-                ("quant_err", ctypes.c_void_p)]
+                ("quant_err", ctypes.c_void_p), ("row_cuts", ctypes.c_void_p)]
 
 
 class MaHyper(ctypes.Structure):
@@ -61,6 +61,8 @@ def _load():
         "ma_param_update": (ci, [i64, vp, vp, f32, ci, f32, ci, vp]),
         "ma_fused_step": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper), vp]),
         "ma_fused_step_check": (ci, [ctypes.POINTER(MaTensor), ctypes.POINTER(MaHyper)]),
+        "ma_fused_step_row_cuts": (ctypes.c_int64, [ctypes.POINTER(MaTensor),
+                                                    ctypes.POINTER(MaHyper)]),
         "ma_fused_step_densified": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
                                          ctypes.c_double, vp]),
         "ma_fused_step_quant_err": (ci, [ctypes.POINTER(MaTensor), ci, ctypes.POINTER(MaHyper),
@@ -95,7 +97,8 @@ EXPORTS = ("ma_error_string", "ma_get_sm_count",
            "ma_get_max_floats_for_shared_memory_per_thread_block", "ma_copy_values",
            "ma_zerorize_block_components", "ma_asymm_block_quant", "ma_asymm_block_quant_inv",
            "ma_compute_microadam_update", "ma_block_topk", "ma_block_minmax", "ma_param_update",
-           "ma_fused_step", "ma_fused_step_check", "ma_fused_step_densified",
+           "ma_fused_step", "ma_fused_step_check", "ma_fused_step_row_cuts",
+           "ma_fused_step_densified",
            "ma_fused_step_quant_err", "ma_logged_step", "ma_logged_step_partials",
            "ma_spanning_step", "ma_spanning_step_static", "ma_spanning_step_workspace",
            "ma_spanning_step_check", "ma_sparse_scalar_products",

@@ -67,6 +67,7 @@ class _Table:
             self.view[name] = [e.st[name].data_ptr() for e in entries]
         self.view['quant_err'] = [e.st['quant_err'].data_ptr() if 'quant_err' in e.st else 0
                                   for e in entries]
+        self.view['row_cuts'] = [0 if e.cuts is None else e.cuts.data_ptr() for e in entries]
         self.view['d'] = [e.st['d'] for e in entries]
         self.view['k'] = [e.st['k'] for e in entries]
 
@@ -81,12 +82,21 @@ class _Table:
 
 class _Entry:
     """What the step knows about one parameter between steps."""
-    __slots__ = ('p', 'st', 'route', 'lr', 'wd', 'p_addr', 'g_addr')
+    __slots__ = ('p', 'st', 'route', 'lr', 'wd', 'p_addr', 'g_addr', 'cuts')
 
     def __init__(self, p, st, route):
         self.p, self.st, self.route = p, st, route
         self.lr = self.wd = 0.0
         self.p_addr = self.g_addr = 0  # device addresses of p and p.grad in the current step
+        # ma_fused_step's cache of where each window row crosses the multiples of 512
+        # coordinates (include/microadam_hip.h, ma_fused_step_row_cuts): not part of the state,
+        # rebuilt row by row after a reload; None when the tensor's step has no use for it
+        self.cuts = None
+
+    def forget_row_cuts(self, row):
+        """Row `row` of the window is being written by something else than ma_fused_step."""
+        if self.cuts is not None:
+            self.cuts[row].fill_(-1)
 
 
 class MicroAdam(torch.optim.Optimizer):
@@ -199,6 +209,11 @@ class MicroAdam(torch.optim.Optimizer):
         e = self._entries.get(p)
         if e is None or e.st is not st or repaired:
             e = self._entries[p] = _Entry(p, st, self._static_route(p, st))
+            if e.route == FUSED:
+                probe, h = self._probe(p, st)
+                words = _hip.lib.ma_fused_step_row_cuts(ctypes.byref(probe), ctypes.byref(h))
+                if words > 0:
+                    e.cuts = torch.full((self.m, words), -1, dtype=torch.int16, device=p.device)
             self._tables.clear()
         return e
 
@@ -216,13 +231,7 @@ class MicroAdam(torch.optim.Optimizer):
                     + int(math.ceil((d - d // dbs * dbs) * self.k_init)))
         if dbs != min(d, self.d_block_size) or st['k'] != expect_k:
             return OP_BY_OP
-        probe = _hip.MaTensor()
-        for name in ('p', 'g'):
-            setattr(probe, name, 256)  # stands for any 16-byte aligned address
-        for name, _ in _TYPED_STATE:
-            setattr(probe, name, st[name].data_ptr())
-        probe.d, probe.k, probe.index = d, st['k'], 0
-        h = self._hyper(p.dtype, max(self.steps, 1))
+        probe, h = self._probe(p, st)
         if _hip.lib.ma_fused_step_check(ctypes.byref(probe), ctypes.byref(h)) == 0:
             if self.alpha == -2:
                 return FUSED_QUANT_ERR
@@ -235,6 +244,17 @@ class MicroAdam(torch.optim.Optimizer):
                                            float(self.alpha)) == 0:
             return SPANNING
         return OP_BY_OP
+
+    def _probe(self, p, st):
+        """A record of p's state (with stand-ins for the buffers of a step) and the
+        hyper-parameters, for the library's admission and size queries."""
+        probe = _hip.MaTensor()
+        for name in ('p', 'g'):
+            setattr(probe, name, 256)  # stands for any 16-byte aligned address
+        for name, _ in _TYPED_STATE:
+            setattr(probe, name, st[name].data_ptr())
+        probe.d, probe.k, probe.index = st['d'], st['k'], 0
+        return probe, self._hyper(p.dtype, max(self.steps, 1))
 
     def _fusable(self, p, st):
         """Route p takes in a step with its current gradient: 0 op by op, 1 fused, 2 spanning,
@@ -349,6 +369,8 @@ class MicroAdam(torch.optim.Optimizer):
                 ws = self._workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
             ws_ptr, ws_len = ws.data_ptr(), ws.numel()
         if sums is not None:
+            for e in entries:  # a logging step's kernels do not file the cuts of the row they write
+                e.forget_row_cuts(e.st['index'])
             need = _hip.lib.ma_logged_step_partials(table.records, n, ctypes.byref(h))
             part = self._partials
             if part is None or part.numel() < need or part.device != device:
@@ -380,7 +402,9 @@ class MicroAdam(torch.optim.Optimizer):
         """One tensor through the reference's own sequence of device operations.  Returns the
         logging sums of this tensor (all zero unless logging_step)."""
         out = dict(norm_qe=0, norm_g=0, norm_u=0, norm_e=0, sparsity_u=0, sparsity_qe=0)
-        st = self._entry(p, lr, wd).st
+        entry = self._entry(p, lr, wd)
+        st = entry.st
+        entry.forget_row_cuts(st['index'])
         acc = p.grad.view(-1)  # the gradient buffer is accumulator, update and scratch in turn
         d, q = st['d'], self.quant_block_size
         error, lo, hi = st['error'], st['min_vals'], st['max_vals']

@@ -32,10 +32,10 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header():
     from ista_daslab_optimizers import _hip
     # struct ma_tensor: 7 pointers, 2 int64, 2 double, 2 int32; struct ma_hyper: see header
-    assert ctypes.sizeof(_hip.MaTensor) == 7 * 8 + 2 * 8 + 2 * 8 + 2 * 4 + 8
+    assert ctypes.sizeof(_hip.MaTensor) == 7 * 8 + 2 * 8 + 2 * 8 + 2 * 4 + 8 + 8
     assert ctypes.sizeof(_hip.MaHyper) == 8 + 4 + 4 + 8 + 8 + 4 * 8
     assert _hip.MaTensor.lr.offset == 72 and _hip.MaTensor.index.offset == 88
-    assert _hip.MaTensor.quant_err.offset == 96
+    assert _hip.MaTensor.quant_err.offset == 96 and _hip.MaTensor.row_cuts.offset == 104
 
 
 def test_host_helpers_mirror_reference():
@@ -93,6 +93,34 @@ def test_step_checks_refuse_what_does_not_fit_in_lds():
         assert _hip.lib.ma_fused_step_check(ctypes.byref(t), ctypes.byref(h)) == want, k_init
         h.quant_block_size = 40960
         assert _hip.lib.ma_spanning_step_check(ctypes.byref(t), ctypes.byref(h), 0.5) == want, k_init
+
+
+def test_row_cuts_query():
+    """Host-only: which tensors ma_fused_step keeps a cache of row cuts for, and its size."""
+    from ista_daslab_optimizers import _hip
+    import math
+    t = _hip.MaTensor()
+    for f in ("p", "g", "error", "min_vals", "max_vals", "I", "V"):
+        setattr(t, f, 0x10000)
+    t.lr, t.weight_decay, t.index = 1e-3, 0.0, 0
+
+    def words(d, m, k_init, dtype=_hip.MA_BF16):
+        dbs = min(d, 20480)
+        t.d = d
+        t.k = d // dbs * int(math.ceil(dbs * k_init)) + int(math.ceil(d % dbs * k_init))
+        h = _hip.MaHyper(1, m, dtype, 64, 20480, k_init, 0.9, 0.999, 1e-8)
+        return _hip.lib.ma_fused_step_row_cuts(ctypes.byref(t), ctypes.byref(h))
+
+    # 20 rows of 1024 entries per block: two launches, 41 cuts for each of the 3 blocks
+    assert words(20480 * 2 + 4096, 20, 0.05) == 3 * 41
+    assert words(20480 * 2, 20, 0.05) == 2 * 41
+    # the window of the 7B configuration fits the one-pass stage
+    assert words(20480 * 2 + 4096, 10, 0.01) == 0
+    # two launches, but rows of at most 512 entries are not listed by coordinate
+    assert words(20480 * 2, 20, 0.01) == 0
+    # a tensor shorter than a top-k block: one block, ceil(d / 512) + 1 cuts
+    assert words(16384, 20, 0.05) == 33
+    assert _hip.lib.ma_fused_step_row_cuts(None, None) == _hip.MA_ERR_ARG
 
 
 def test_logged_step_argument_checks():

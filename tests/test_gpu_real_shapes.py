@@ -85,3 +85,48 @@ def test_outlier_layers_match_oracle_past_the_ring_wrap(oracle):
 def test_llama3_8b_layers_match_oracle(oracle):
     _run(oracle, [(4096, 4096), (1024, 4096)], 10, 100000, 0.01, 0.5, 12, {1, 2, 10, 11, 12}, 2,
          "normal")
+
+
+def test_row_cuts_cache_survives_route_changes_and_reloads(oracle):
+    """Dense windows (20 rows of 1024 entries per block) are stepped in two launches, the second
+    of which reads where every row crosses the multiples of 512 coordinates from a cache the
+    first one fills (ma_fused_step_row_cuts).  Steps taken op by op in between, and a reloaded
+    state, leave rows the cache does not know: results stay those of the oracle, bit for bit."""
+    from ista_daslab_optimizers import MicroAdam
+    shapes = [(20480 * 3 + 5000,), (16384,), (2048, 30)]
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    start = [(torch.randn(s, generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+             for s in shapes]
+    oparams = [to_np(p).reshape(-1) for p in start]
+    oref = oracle.OracleMicroAdam(oparams, 20, 1e-3, 32, 0.05, 0.0, d_block_size=20480)
+    params = [torch.nn.Parameter(p.clone()) for p in start]
+
+    def make():
+        return MicroAdam(params, m=20, lr=1e-3, quant_block_size=32, k_init=0.05, alpha=0.0)
+
+    opt = make()
+    for s in range(27):
+        grads = [_normal(shp, gen, 1e-3) for shp in shapes]
+        host = [to_np(g).reshape(-1) for g in grads]
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.use_fused = s not in (4, 5, 23)       # those steps go op by op
+        if s == 9:                                # a reload drops the cache
+            sd = opt.state_dict()
+            opt = make()
+            opt.load_state_dict(sd)
+        opt.step()
+        oref.step(host)
+        entry = opt._entries[params[0]]
+        if s == 0:
+            assert entry.cuts is not None and entry.cuts.shape == (20, 4 * 41)
+            assert opt._entries[params[1]].cuts.shape == (20, 33)
+        row = (opt.state[params[0]]["index"] - 1) % 20
+        known = bool((entry.cuts[row, ::41] == 0).all())
+        assert known == opt.use_fused, f"step {s + 1}: row {row} of the cache"
+        for i, p in enumerate(params):
+            ctx = f"step {s + 1} tensor {i}"
+            got = to_np(p.data).reshape(-1)
+            assert np.array_equal(got, oparams[i]), ctx
+            if s + 1 in (1, 6, 10, 21, 24, 27):
+                assert_state_equal(opt.state[p], oref.state[i], ctx)
