@@ -105,6 +105,7 @@ struct FusedParams {
 constexpr int kAuxLog = 1, kAuxQuantErr = 2;
 constexpr int kSpanWords = 8;  // workspace words per top-k block of the two-pass route
 constexpr int kRowCutStep = 512;  // coordinates between two cuts of a window row
+constexpr int kHintLongRow = 4 * 512;  // longest block row whose previous threshold is looked up
 
 // Layout of a tensor's cache of row cuts: (row, block, cut) -> word
 struct RowCuts {
@@ -387,9 +388,12 @@ struct FusedBlock {
     __device__ __forceinline__ void load_hint(const BlockGeo &G) {
         hint = 0x7fffu;
         if constexpr (FULL && R::kBF16) {
-            if (tid < G.kb && G.kb <= kWG) {
-                const int prev = (G.D.row == 0 ? P.W.rows_total : G.D.row) - 1;
-                hint = G.D.V[(int64_t)prev * G.D.k + G.col0 + tid] & 0x7fffu;
+            const int prev = (G.D.row == 0 ? P.W.rows_total : G.D.row) - 1;
+            const uint16_t *Vp = G.D.V + ((int64_t)prev * G.D.k + G.col0);
+            if (G.kb <= kWG) {
+                if (tid < G.kb) hint = Vp[tid] & 0x7fffu;
+            } else if (G.kb <= kHintLongRow) {
+                for (int j = tid; j < G.kb; j += kWG) hint = min(hint, Vp[j] & 0x7fffu);
             }
         }
     }
@@ -510,7 +514,13 @@ struct FusedBlock {
         if (!topk_done) {
             uint32_t T;
             int take_eq;
-            select_threshold(r, kb, hist, sh, T, take_eq, P.L.hist_log2);
+            bool have = false;
+            if constexpr (FULL && R::kBF16) {
+                // block rows too long for the candidate lists: the hint gives the threshold
+                if (kb > kWG && kb <= kHintLongRow)
+                    have = hint_threshold_bf16(r, kb, hint, hist, sh, T, take_eq);
+            }
+            if (!have) select_threshold(r, kb, hist, sh, T, take_eq, P.L.hist_log2);
             launder(r);
             compact_selected(r, T, take_eq, kb, sel_idx, sel_val, sh);
             launder(r);

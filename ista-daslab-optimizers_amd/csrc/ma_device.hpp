@@ -483,12 +483,16 @@ __device__ __forceinline__ uint32_t select_kth_key15(const uint32_t (&v)[N], uin
 // min(key - base, 255), so every bin below 255 is one key value.  Returns the kb-th largest key
 // as select_kth_key15 does, or 0xffffffff if it fell into the bin of the keys base + 255 and
 // above (then nothing else is valid either).  hist: 257 * kSmallCopies zero words; shp: 2 words.
+__device__ __forceinline__ uint32_t walk_near_bins(int kb, uint32_t base, const uint32_t *hist,
+                                                   uint32_t *shp, uint32_t *sh_neq, int &take_eq,
+                                                   int &n_eq);
+
 template <int N>
 __device__ __forceinline__ uint32_t select_kth_near(const uint32_t (&v)[N], uint32_t valid,
                                                     int kb, uint32_t base, uint32_t *hist,
                                                     uint32_t *shp, uint32_t *sh_neq,
                                                     int &take_eq, int &n_eq) {
-    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    const int tid = opaque_tid(), lane = tid & 63;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const uint32_t off = v[i] - base;
@@ -496,6 +500,15 @@ __device__ __forceinline__ uint32_t select_kth_near(const uint32_t (&v)[N], uint
         atomicAdd(&hist[bin * kSmallCopies + (lane & (kSmallCopies - 1))], 1u);
     }
     __syncthreads();
+    return walk_near_bins(kb, base, hist, shp, sh_neq, take_eq, n_eq);
+}
+
+// Second half of select_kth_near: the bins are filled (and a barrier has passed); wave 0 walks
+// them from the top.  shp[0] must hold 255 beforehand if fewer than kb keys may have been counted.
+__device__ __forceinline__ uint32_t walk_near_bins(int kb, uint32_t base, const uint32_t *hist,
+                                                   uint32_t *shp, uint32_t *sh_neq, int &take_eq,
+                                                   int &n_eq) {
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     if (wave == 0) {
         uint32_t c[4], tot = 0;
 #pragma unroll
@@ -637,6 +650,59 @@ __device__ __forceinline__ bool hint_topk_bf16(R &r, int kb, uint32_t hint, uint
                                        (uint32_t)kb, hist,
                                        reinterpret_cast<uint16_t *>(hist + 2 * kSmallHistWords),
                                        L);
+}
+
+// The threshold of a full bf16 block's kb largest magnitudes from a lower bound known
+// beforehand, for selections too long for the candidate lists of hint_topk_bf16 (which then
+// take compact_selected).  `hint` as there.  The elements with key >= L are counted by key - L,
+// straight from the registers, in the bins of select_kth_near; true with (T, take_eq) as
+// select_threshold gives them, false (uniformly) if fewer than kb elements reach L, the kb-th
+// largest lies 255 key steps or more above L, or there is no usable hint.  Any hint gives the
+// same threshold or a refusal.  hist: 257 * kSmallCopies words; sh: the kSh* words.
+template <class R>
+__device__ __forceinline__ bool hint_threshold_bf16(const R &r, int kb, uint32_t hint,
+                                                    uint32_t *hist, uint32_t *sh, uint32_t &T,
+                                                    int &take_eq) {
+    constexpr int C = R::kC;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    const uint32_t wmin = wave_min_to_last(hint);
+    if (lane == kWave - 1) sh[kShScan + wave] = wmin;
+    for (int i = tid; i < 257 * kSmallCopies; i += kWG) hist[i] = 0;
+    if (tid == 0) {
+        sh[kShSel] = 255u;  // stays if fewer than kb elements are counted
+        sh[kShSel + 1] = 0u;
+    }
+    __syncthreads();
+    uint32_t hmin = 0x7fffu;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) hmin = min(hmin, sh[kShScan + w]);
+    const float lf = __uint_as_float(hmin << 16) * 0.96875f;
+    const uint32_t L = __float_as_uint(lf) >> 16;
+    bool usable = L != 0 && hmin != 0x7fffu;  // (a fresh window's rows are all zero)
+    if (usable) {
+        const uint32_t LL = L | L << 16;
+        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+        uint32_t *mine = hist + (lane & (kSmallCopies - 1));
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // per 16-bit half: (key | 0x8000) - L has bit 15 set exactly when key >= L, and
+                // then key - L below it
+                const us2 a = __builtin_bit_cast(us2, (r.w[c][i] & 0x7fff7fffu) | 0x80008000u);
+                const uint32_t t = __builtin_bit_cast(uint32_t, (us2)(a - __builtin_bit_cast(us2, LL)));
+                if (t & 0x8000u) atomicAdd(mine + min(t & 0x7fffu, 255u) * kSmallCopies, 1u);
+                if (t & 0x80000000u)
+                    atomicAdd(mine + min((t >> 16) & 0x7fffu, 255u) * kSmallCopies, 1u);
+            }
+        }
+    }
+    __syncthreads();
+    int n_eq;
+    const uint32_t found =
+        walk_near_bins(kb, L, hist, sh + kShSel, sh + kShNEq, take_eq, n_eq);
+    T = found;
+    return usable && found != 0xffffffffu;
 }
 
 // The fast top-k of a full bf16 block.  `park` (kRound*C uint16 cells) receives the block;
