@@ -510,13 +510,22 @@ struct FusedBlock {
                 slot_clear = topk_done && P.L.slot_cells == C * kRound;
             }
         }
-        row_sorted = !topk_done;  // the general selection lists its entries by coordinate
+        row_sorted = !topk_done;  // the selections below list their entries by coordinate
+        if constexpr (FULL && R::kBF16) {
+            // block rows too long for the candidate lists, where the LDS plan has the cells to
+            // park the block in: threshold and ordered selection from the hint
+            if (kb > kWG && kb <= kHintLongRow && P.L.cell_bytes == 2 &&
+                P.L.slot_cells >= C * kRound) {
+                topk_done = hint_sorted_topk_bf16(r, kb, hint, cell16, hist, sh, sel_idx, sel_val);
+                launder(r);
+            }
+        }
         if (!topk_done) {
             uint32_t T;
             int take_eq;
             bool have = false;
             if constexpr (FULL && R::kBF16) {
-                // block rows too long for the candidate lists: the hint gives the threshold
+                // (without the cells: the hint gives the threshold at least)
                 if (kb > kWG && kb <= kHintLongRow)
                     have = hint_threshold_bf16(r, kb, hint, hist, sh, T, take_eq);
             }

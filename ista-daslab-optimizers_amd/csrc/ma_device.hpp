@@ -705,6 +705,166 @@ __device__ __forceinline__ bool hint_threshold_bf16(const R &r, int kb, uint32_t
     return usable && found != 0xffffffffu;
 }
 
+// Flags of the elements of a register-resident bf16 block whose key is at least `bound` (a
+// 15-bit key, or 0x8000 for "none").  Byte B of `lo` holds, for chunk c = 0..3, element B at bit
+// 2c and element 4 + B at bit 2c + 1; `hi` the same for the chunks above.
+template <class R>
+__device__ __forceinline__ void flags_at_least(const R &r, uint32_t bound, uint32_t &lo,
+                                               uint32_t &hi) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    static_assert(R::kC <= 8, "two words of flags");
+    const uint32_t BB = bound | bound << 16;
+    lo = hi = 0;
+#pragma unroll
+    for (int c = 0; c < R::kC; ++c) {
+        uint32_t t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // per 16-bit half: bit 15 of (key | 0x8000) - bound says key >= bound
+            const us2 a = __builtin_bit_cast(us2, (r.w[c][i] & 0x7fff7fffu) | 0x80008000u);
+            t[i] = __builtin_bit_cast(uint32_t, (us2)(a - __builtin_bit_cast(us2, BB)));
+        }
+        // the bytes whose top bits are the flags: elements 0..3 -> x, elements 4..7 -> y
+        const uint32_t x = __builtin_amdgcn_perm(t[1], t[0], 0x07050301u) & 0x80808080u;
+        const uint32_t y = __builtin_amdgcn_perm(t[3], t[2], 0x07050301u) & 0x80808080u;
+        const uint32_t z = (x >> 7) | (y >> 6);
+        if (c < 4) lo |= z << (2 * c);
+        else hi |= z << (2 * (c - 4));
+    }
+}
+
+// The block top-k of a full bf16 block with a lower bound known beforehand (as hint_topk_bf16
+// takes it), for selections too long for candidate lists, and with the entries listed by
+// increasing coordinate, which is the order compact_selected gives and window_param_kernel
+// relies on.  The block is parked in `park` (kRound * C uint16 cells); the elements with key >= L
+// are counted by key - L in the bins of select_kth_near (one turn per flagged element of a
+// lane, so a few turns instead of one step per element); with the threshold T known, every
+// lane ranks its own elements >= T from the flags alone (counts per chunk, a scan over the
+// lanes per chunk, the waves' totals), moves the selected ones to sel_idx / sel_val and clears
+// them in the parked block, from which r is read back.  Ties at T go to the lowest coordinates.
+// False (uniformly, r unchanged) if fewer than kb elements reach L, the kb-th largest lies 255
+// key steps or more above L, or there is no usable hint; any hint gives the same selection or a
+// refusal.  hist: 257 * kSmallCopies words; sh: the kSh* words.  Ends with a barrier.
+template <class R>
+__device__ __forceinline__ bool hint_sorted_topk_bf16(R &r, int kb, uint32_t hint, uint16_t *park,
+                                                      uint32_t *hist, uint32_t *sh,
+                                                      uint16_t *sel_idx, uint16_t *sel_val) {
+    constexpr int C = R::kC;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    const uint32_t wmin = wave_min_to_last(hint);
+    if (lane == kWave - 1) sh[kShScan + wave] = wmin;
+    for (int i = tid; i < 257 * kSmallCopies; i += kWG) hist[i] = 0;
+    if (tid == 0) {
+        sh[kShSel] = 255u;  // stays if fewer than kb elements are counted
+        sh[kShSel + 1] = 0u;
+    }
+    __syncthreads();
+    uint32_t hmin = 0x7fffu;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) hmin = min(hmin, sh[kShScan + w]);
+    const float lf = __uint_as_float(hmin << 16) * 0.96875f;
+    const uint32_t L = __float_as_uint(lf) >> 16;
+    if (L == 0 || hmin == 0x7fffu) return false;  // (a fresh window's rows are all zero)
+
+    const int off0 = chunk_off<C>(wave, 0, lane);
+    // element behind flag bit b of the low / high word: chunk, then offset in the block
+    auto offset_of = [&](int b, bool low) {
+        const int c = ((b >> 1) & 3) + (low ? 0 : 4);
+        const int e = (b >> 3) + 4 * (b & 1);
+        return off0 + c * (kWave * kChunk) + e;
+    };
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+        *reinterpret_cast<uint4 *>(park + chunk_off<C>(wave, c, lane)) =
+            make_uint4(r.w[c][0], r.w[c][1], r.w[c][2], r.w[c][3]);
+    uint32_t flo, fhi;
+    flags_at_least(r, L, flo, fhi);
+    uint32_t *mine = hist + (lane & (kSmallCopies - 1));
+    while (__builtin_amdgcn_ballot_w64((flo | fhi) != 0) != 0) {
+        const bool low = flo != 0;
+        const uint32_t f = low ? flo : fhi;
+        if (f != 0) {
+            const int b = __ffs(f) - 1;
+            if (low) flo &= flo - 1;
+            else fhi &= fhi - 1;
+            const uint32_t key = park[offset_of(b, low)] & 0x7fffu;  // (the lane's own cell)
+            atomicAdd(mine + min(key - L, 255u) * kSmallCopies, 1u);
+        }
+    }
+    __syncthreads();
+    int take_eq, n_eq;
+    const uint32_t T = walk_near_bins(kb, L, hist, sh + kShSel, sh + kShNEq, take_eq, n_eq);
+    if (T == 0xffffffffu) return false;
+
+    // ---- flags of the elements >= T and of those == T; their counts before every lane's chunk
+    uint32_t glo, ghi, alo, ahi;
+    flags_at_least(r, T, glo, ghi);
+    flags_at_least(r, T + 1u, alo, ahi);
+    const uint32_t qlo = glo & ~alo, qhi = ghi & ~ahi;  // == T
+    uint32_t pre[C];  // low 16: entries >= T before this lane's chunk; high 16: == T
+    uint32_t run = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const uint32_t m = 0x03030303u << (2 * (c & 3));
+        const uint32_t cnt = (uint32_t)__popc((c < 4 ? glo : ghi) & m) +
+                             ((uint32_t)__popc((c < 4 ? qlo : qhi) & m) << 16);
+        const uint32_t incl = wave_incl_scan(cnt, lane);
+        pre[c] = run + incl - cnt;
+        run += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    }
+    if (lane == 0) sh[kShScan + wave] = run;
+    __syncthreads();
+    uint32_t base = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+        if (w < wave) base += sh[kShScan + w];
+
+    // ---- one turn per selected candidate of a lane: its rank from the flags below it
+    uint32_t tlo = glo, thi = ghi;
+    while (__builtin_amdgcn_ballot_w64((tlo | thi) != 0) != 0) {
+        const bool low = tlo != 0;
+        const uint32_t f = low ? tlo : thi;
+        if (f != 0) {
+            const int b = __ffs(f) - 1;
+            if (low) tlo &= tlo - 1;
+            else thi &= thi - 1;
+            const int cq = (b >> 1) & 3, c = cq + (low ? 0 : 4), B = b >> 3;
+            // flags of the same chunk of this lane with lower coordinates: elements 0..3 sit at
+            // bit 2 cq of the bytes, elements 4..7 one bit above
+            const uint32_t firsts = 0x01010101u << (2 * cq), seconds = firsts << 1;
+            const uint32_t bytes_below = (1u << (8 * B)) - 1u;
+            const uint32_t below = (b & 1) ? (firsts | (seconds & bytes_below))
+                                           : (firsts & bytes_below);
+            uint32_t p = pre[0];
+#pragma unroll
+            for (int k = 1; k < C; ++k) p = c == k ? pre[k] : p;
+            p += base;
+            const uint32_t ge_word = low ? glo : ghi, eq_word = low ? qlo : qhi;
+            const uint32_t ge_before = (p & 0xffffu) + (uint32_t)__popc(ge_word & below);
+            const uint32_t eq_before = (p >> 16) + (uint32_t)__popc(eq_word & below);
+            const bool is_eq = ((eq_word >> b) & 1u) != 0;
+            const bool sel = !is_eq || eq_before < (uint32_t)take_eq;
+            const uint32_t pos = (ge_before - eq_before) + min(eq_before, (uint32_t)take_eq);
+            if (sel && pos < (uint32_t)kb) {
+                const int off = offset_of(b, low);
+                sel_idx[pos] = (uint16_t)off;
+                sel_val[pos] = park[off];
+                park[off] = 0;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(park + chunk_off<C>(wave, c, lane));
+        r.w[c][0] = q.x;
+        r.w[c][1] = q.y;
+        r.w[c][2] = q.z;
+        r.w[c][3] = q.w;
+    }
+    return true;
+}
+
 // The fast top-k of a full bf16 block.  `park` (kRound*C uint16 cells) receives the block;
 // on success (returns true, uniformly) sel_idx / sel_val hold the kb selected entries, largest
 // magnitude first, the selected cells are zeroed, and r is reloaded from `park`.  On false

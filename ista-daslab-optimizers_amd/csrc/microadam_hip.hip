@@ -374,7 +374,7 @@ static LdsMap plan_lds(int dbs_max, int kb_max, int m, int elem_bytes, bool one_
 // LDS plan of a block kernel that ends with the quantisation: the selection's needs only (the
 // cells are where the fast selection parks the block; longer block rows take the general
 // selection, which leaves the block in registers).
-static LdsMap plan_lds_select_only(int dbs_max, int kb_max) {
+static LdsMap plan_lds_select_only(int dbs_max, int kb_max, int elem_bytes) {
     LdsMap L;
     memset(&L, 0, sizeof L);
     L.off_sel_idx = kMiscBytes;
@@ -382,9 +382,23 @@ static LdsMap plan_lds_select_only(int dbs_max, int kb_max) {
     L.off_slot = L.off_sel_val + align16(kb_max * 2);
     L.slot_cells = (dbs_max + 7) & ~7;
     L.cell_bytes = 2;
-    L.off_union = L.off_slot + (kb_max <= kWG ? align16(L.slot_cells * 2) : 0);
-    L.hist_log2 = 5;
-    L.total = L.off_union + kHistBytes;
+    if (kb_max <= kWG) {
+        L.off_union = L.off_slot + align16(L.slot_cells * 2);
+        L.hist_log2 = 5;
+        L.total = L.off_union + kHistBytes;
+    } else if (elem_bytes == 2 && kb_max <= kHintLongRow) {
+        // the hinted ordered selection parks the block too; the general selection, which is
+        // then the exception, makes do with 4 copies of its histogram, and the whole stays
+        // within a third of the LDS
+        L.off_union = L.off_slot + align16(L.slot_cells * 2);
+        L.hist_log2 = 2;
+        L.total = L.off_union + ((257 << L.hist_log2) * 4);
+    } else {
+        L.slot_cells = 0;
+        L.off_union = L.off_slot;
+        L.hist_log2 = 5;
+        L.total = L.off_union + kHistBytes;
+    }
     return L;
 }
 
@@ -907,7 +921,7 @@ static int step_impl(const ma_tensor *tensors, int n_tensors, const ma_hyper *h,
                 // a window too large for the one-pass stage: the block kernel ends with the
                 // quantisation, a second launch over the same blocks forms the update
                 P.win_apart = 1;
-                P.L = plan_lds_select_only(dbs_max, kb_max);
+                P.L = plan_lds_select_only(dbs_max, kb_max, elem_bytes);
                 plan.back().kind = kBlockPart;
                 PlannedLaunch second = plan.back();
                 second.kind = kWindowPart;
