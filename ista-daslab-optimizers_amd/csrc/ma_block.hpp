@@ -30,9 +30,10 @@ constexpr int kFastTopkBytes = (2 * kSmallHistWords + 512) * 4;
 constexpr int kHistBytes =
     257 * kHistCopies * 4 > kFastTopkBytes ? 257 * kHistCopies * 4 : kFastTopkBytes;
 
+constexpr int kWindowPad = 16;  // zero weights behind the last row, for code that reads rows in batches
 struct WindowWeights {
-    float w1[kMaxWindow];
-    float w2[kMaxWindow];
+    float w1[kMaxWindow + kWindowPad];
+    float w2[kMaxWindow + kWindowPad];
     float s1, s2, eps;
     int rows;        // live rows: min(t, m)
     int rows_total;  // m
@@ -2486,23 +2487,29 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
                 //      nothing between the requests waits for an answer.
                 uint32_t ei[kWinRowBatch], ev[kWinRowBatch];
                 float w1[kWinRowBatch], w2[kWinRowBatch];
+                uint32_t at[kWinRowBatch], e2[kWinRowBatch];
                 uint32_t longer = 0;  // bit i: row r0 + i has more than 64 entries in the chunk
                 const int *tp = table + r0 * stride + ch;
+                static_assert(kWinRowBatch <= kWindowPad, "weights are read past the last row");
+                // (nothing below depends on anything loaded above it, and nothing branches)
+#pragma unroll
+                for (int i = 0; i < kWinRowBatch; ++i) {
+                    at[i] = (uint32_t)tp[i * stride] + lane2;
+                    e2[i] = (uint32_t)tp[i * stride + 1];
+                    w1[i] = P.W.w1[r0 + i];  // (zero behind the last row)
+                    w2[i] = P.W.w2[r0 + i];
+                }
 #pragma unroll
                 for (int i = 0; i < kWinRowBatch; ++i) {
                     const bool live = r0 + i < rows;
                     const int r = live ? r0 + i : 0;
-                    w1[i] = live ? P.W.w1[r] : 0.0f;
-                    w2[i] = live ? P.W.w2[r] : 0.0f;
-                    const uint32_t at = (uint32_t)tp[i * stride] + lane2;
-                    const uint32_t e2 = (uint32_t)tp[i * stride + 1];
-                    if (live && __builtin_amdgcn_ballot_w64(at + 2u * kWave < e2) != 0)
-                        longer |= 1u << i;
+                    const bool more = __builtin_amdgcn_ballot_w64(at[i] + 2u * kWave < e2[i]) != 0;
+                    longer |= (live && more ? 1u : 0u) << i;
                     const uint32_t bytes = live ? 2u * (uint32_t)kb : 0u;
                     const __amdgpu_buffer_rsrc_t bi = byte_buffer(Ib + (int64_t)r * k, bytes);
                     const __amdgpu_buffer_rsrc_t bv = byte_buffer(Vb + (int64_t)r * k, bytes);
-                    ei[i] = __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at, 0, 0);
-                    ev[i] = __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at, 0, 0);
+                    ei[i] = __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at[i], 0, 0);
+                    ev[i] = __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at[i], 0, 0);
                 }
                 // ---- then the sums, row after row.  An entry of a later chunk goes to the
                 //      spare cell; one past the row (index 0, value 0) adds 0 to the first cell
@@ -2525,17 +2532,17 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
                     if ((longer >> i) & 1u) {  // the rest of the stretch, before the next row
                         const int r = r0 + i;
                         const uint32_t s2 = (uint32_t)tp[i * stride];
-                        const uint32_t e2 = (uint32_t)tp[i * stride + 1];
+                        const uint32_t end = (uint32_t)tp[i * stride + 1];
                         const __amdgpu_buffer_rsrc_t bi =
                             byte_buffer(Ib + (int64_t)r * k, 2u * (uint32_t)kb);
                         const __amdgpu_buffer_rsrc_t bv =
                             byte_buffer(Vb + (int64_t)r * k, 2u * (uint32_t)kb);
-                        for (uint32_t a2 = s2 + 2u * kWave; a2 < e2; a2 += 2u * kWave) {
-                            const uint32_t at = a2 + lane2;
+                        for (uint32_t a2 = s2 + 2u * kWave; a2 < end; a2 += 2u * kWave) {
+                            const uint32_t a3 = a2 + lane2;
                             const uint32_t idx =
-                                __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at, 0, 0);
+                                __builtin_amdgcn_raw_buffer_load_b16(bi, (int)a3, 0, 0);
                             const uint32_t vb =
-                                __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at, 0, 0);
+                                __builtin_amdgcn_raw_buffer_load_b16(bv, (int)a3, 0, 0);
                             add(idx, vb);
                         }
                     }
