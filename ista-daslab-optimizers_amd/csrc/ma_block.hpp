@@ -2435,9 +2435,15 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
         }
     }
     }
+    // (the batches below read up to kWindowPad rows past the live ones: empty stretches)
+    for (int i = rows * stride + tid; i < (rows + kWindowPad) * stride; i += kWG) table[i] = 0;
     if (bad) atomicOr(&sh[0], 1u);
     __syncthreads();
-    const bool in_order = sh[0] == 0;
+    // One buffer per array for all rows of the block's stretch of the window, the row chosen by
+    // a scalar byte offset: possible while the rows from this block's first entry to its
+    // stretch of the last row span less than 4 GiB.
+    const uint64_t span_bytes = ((uint64_t)(P.W.rows_total - 1) * (uint64_t)k + (uint64_t)kb) * 2u;
+    const bool in_order = sh[0] == 0 && span_bytes <= 0xffffffffull;
     // table[row][ch]: byte offset of the first entry of chunk ch in the row's stretch of the
     // block
 
@@ -2467,6 +2473,10 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
         constexpr int kPerLane = kWinChunk / kWave;  // coordinates of a chunk per lane
         float2 *z = reinterpret_cast<float2 *>(sums) + wave * (kWinChunk + 8);
         const uint32_t lane2 = (uint32_t)lane * 2u;
+        const __amdgpu_buffer_rsrc_t all_i = byte_buffer(Ib, (uint32_t)span_bytes);
+        const __amdgpu_buffer_rsrc_t all_v = byte_buffer(Vb, (uint32_t)span_bytes);
+        const int row_stride = (int)(uint32_t)(2 * k);  // bytes from a row to the next
+        const int last_row = P.W.rows_total - 1;
         for (int ch = wave; ch < nch; ch += kWaves) {
             const int base = ch * kWinChunk, off = base + lane * kPerLane;
             RawChunk<R> praw[kPerLane / kChunk];
@@ -2478,20 +2488,26 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
             for (int i = 0; i < kPerLane / 2; ++i)
                 reinterpret_cast<float4 *>(z + lane * kPerLane)[i] = zero4;
             __builtin_amdgcn_wave_barrier();
+            // rows with more than 64 entries in this chunk (bit r), found once for the chunk
+            uint64_t long_rows = 0;
+            {
+                int len = 0;
+                if (lane < rows) len = table[lane * stride + ch + 1] - table[lane * stride + ch];
+                long_rows = __builtin_amdgcn_ballot_w64(len > 2 * kWave);
+            }
             for (int r0 = 0; r0 < rows; r0 += kWinRowBatch) {
-                // ---- all requests of the batch first: entry s + lane of every row's stretch.
-                //      Entries past the stretch (they belong to later chunks) or past the row
-                //      (the buffer returns index 0, value 0 for them) are sorted out when they
-                //      are added.  A batch that reaches past the last live row reads those rows
-                //      through buffers of no bytes, with weights 0: straight-line code, so that
-                //      nothing between the requests waits for an answer.
+                // ---- all requests of the batch first: entry s + lane of every row's stretch,
+                //      through one buffer per array with the row as a scalar offset.  Lanes
+                //      past the stretch's end (their entries belong to later chunks, blocks or
+                //      rows) are sorted out when the sums are formed; the rows behind the last
+                //      live one have empty stretches and zero weights and are read from the
+                //      last row.  Straight-line code: nothing between the requests waits for
+                //      an answer.
                 uint32_t ei[kWinRowBatch], ev[kWinRowBatch];
                 float w1[kWinRowBatch], w2[kWinRowBatch];
                 uint32_t at[kWinRowBatch], e2[kWinRowBatch];
-                uint32_t longer = 0;  // bit i: row r0 + i has more than 64 entries in the chunk
                 const int *tp = table + r0 * stride + ch;
-                static_assert(kWinRowBatch <= kWindowPad, "weights are read past the last row");
-                // (nothing below depends on anything loaded above it, and nothing branches)
+                static_assert(kWinRowBatch <= kWindowPad, "weights and table rows past the last");
 #pragma unroll
                 for (int i = 0; i < kWinRowBatch; ++i) {
                     at[i] = (uint32_t)tp[i * stride] + lane2;
@@ -2501,24 +2517,20 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
                 }
 #pragma unroll
                 for (int i = 0; i < kWinRowBatch; ++i) {
-                    const bool live = r0 + i < rows;
-                    const int r = live ? r0 + i : 0;
-                    const bool more = __builtin_amdgcn_ballot_w64(at[i] + 2u * kWave < e2[i]) != 0;
-                    longer |= (live && more ? 1u : 0u) << i;
-                    const uint32_t bytes = live ? 2u * (uint32_t)kb : 0u;
-                    const __amdgpu_buffer_rsrc_t bi = byte_buffer(Ib + (int64_t)r * k, bytes);
-                    const __amdgpu_buffer_rsrc_t bv = byte_buffer(Vb + (int64_t)r * k, bytes);
-                    ei[i] = __builtin_amdgcn_raw_buffer_load_b16(bi, (int)at[i], 0, 0);
-                    ev[i] = __builtin_amdgcn_raw_buffer_load_b16(bv, (int)at[i], 0, 0);
+                    const int r = min(r0 + i, last_row);
+                    const int row_bytes = r * row_stride;  // (below 4 GiB, see span_bytes)
+                    // (a lane past the stretch may point past the buffer: it reads 0 then)
+                    ei[i] = __builtin_amdgcn_raw_buffer_load_b16(all_i, (int)at[i], row_bytes, 0);
+                    ev[i] = __builtin_amdgcn_raw_buffer_load_b16(all_v, (int)at[i], row_bytes, 0);
                 }
-                // ---- then the sums, row after row.  An entry of a later chunk goes to the
-                //      spare cell; one past the row (index 0, value 0) adds 0 to the first cell
-                //      or goes there too; +-0 values change nothing anywhere (the rows of a fresh window
-                //      are all (0, 0), and a coordinate counts as named when a sum is not zero).
+                // ---- then the sums, row after row.  What a lane past its stretch's end has
+                //      read goes to the spare cell; +-0 values change nothing anywhere (the rows
+                //      of a fresh window are all (0, 0), and a coordinate counts as named when a
+                //      sum is not zero).
 #pragma unroll
                 for (int i = 0; i < kWinRowBatch; ++i) {
-                    auto add = [&](uint32_t idx, uint32_t vb) {
-                        const uint32_t c = min(idx - (uint32_t)base, (uint32_t)kWinChunk);
+                    auto add = [&](uint32_t idx, uint32_t vb, bool mine) {
+                        const uint32_t c = mine ? idx - (uint32_t)base : (uint32_t)kWinChunk;
                         const float v = bf2f(vb);
                         const float t1 = w1[i] * v;
                         const float vv = v * v;
@@ -2528,22 +2540,16 @@ __global__ __launch_bounds__(kWG, MIN_WAVES) void window_param_kernel(FusedParam
                         x.y = x.y + t2;
                         z[c] = x;
                     };
-                    add(ei[i], ev[i]);
-                    if ((longer >> i) & 1u) {  // the rest of the stretch, before the next row
-                        const int r = r0 + i;
-                        const uint32_t s2 = (uint32_t)tp[i * stride];
-                        const uint32_t end = (uint32_t)tp[i * stride + 1];
-                        const __amdgpu_buffer_rsrc_t bi =
-                            byte_buffer(Ib + (int64_t)r * k, 2u * (uint32_t)kb);
-                        const __amdgpu_buffer_rsrc_t bv =
-                            byte_buffer(Vb + (int64_t)r * k, 2u * (uint32_t)kb);
-                        for (uint32_t a2 = s2 + 2u * kWave; a2 < end; a2 += 2u * kWave) {
-                            const uint32_t a3 = a2 + lane2;
+                    add(ei[i], ev[i], at[i] < e2[i]);
+                    if ((long_rows >> (r0 + i)) & 1u) {  // the rest of the stretch, before the next row
+                        const int row_bytes = (r0 + i) * row_stride;
+                        const uint32_t end = e2[i];
+                        for (uint32_t a2 = at[i] + 2u * kWave; a2 < end; a2 += 2u * kWave) {
                             const uint32_t idx =
-                                __builtin_amdgcn_raw_buffer_load_b16(bi, (int)a3, 0, 0);
+                                __builtin_amdgcn_raw_buffer_load_b16(all_i, (int)a2, row_bytes, 0);
                             const uint32_t vb =
-                                __builtin_amdgcn_raw_buffer_load_b16(bv, (int)a3, 0, 0);
-                            add(idx, vb);
+                                __builtin_amdgcn_raw_buffer_load_b16(all_v, (int)a2, row_bytes, 0);
+                            add(idx, vb, true);
                         }
                     }
                 }

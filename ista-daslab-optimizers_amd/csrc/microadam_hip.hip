@@ -408,9 +408,8 @@ static LdsMap plan_lds_window_param(int dbs_max, int m) {
     memset(&L, 0, sizeof L);
     L.off_slot = kMiscBytes;
     L.slot_cells = (dbs_max + kWinChunk - 1) / kWinChunk + 1;
-    L.off_union = L.off_slot + align16(m * L.slot_cells * 4);  // (a batch may read, and ignore,
-                                                               // table rows past the last: they
-                                                               // lie in the sums)
+    // (the row batches read up to kWindowPad table rows past the last one: kept empty)
+    L.off_union = L.off_slot + align16((m + kWindowPad) * L.slot_cells * 4);
     L.total = L.off_union + kWaves * (kWinChunk + 8) * 8;  // (above the general form's 32 KiB)
     return L;
 }
