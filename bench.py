@@ -27,11 +27,11 @@ CAL_BYTES = 26214 * 40960  # --copy-calibration: bytes the known-size copy reads
 # counters read for a plain copy of known size; (workload, op_by_op) -> bytes.  The figures and
 # the commands behind them are in profiles/.
 MEASURED_TRAFFIC = {
-    ("llama2-7b", False): (50.594e9, "profiles/fused_step_llama2-7b_hbm_traffic.txt"),
-    ("gpt2-small", False): (0.938e9, "profiles/fused_step_gpt2-small_hbm_traffic.txt"),
-    ("outlier-1.3b", False): (17.320e9, "profiles/fused_step_outlier-1.3b_hbm_traffic.txt"),
-    ("llama3-8b", False): (92.067e9, "profiles/spanning_step_llama3-8b_hbm_traffic.txt"),
-    ("llama2-7b-q100k", False): (49.987e9, "profiles/spanning_step_llama2-7b-q100k_hbm_traffic.txt"),
+    ("llama2-7b", False): (50.596e9, "profiles/fused_step_llama2-7b_hbm_traffic.txt"),
+    ("gpt2-small", False): (0.939e9, "profiles/fused_step_gpt2-small_hbm_traffic.txt"),
+    ("outlier-1.3b", False): (15.743e9, "profiles/fused_step_outlier-1.3b_hbm_traffic.txt"),
+    ("llama3-8b", False): (92.069e9, "profiles/spanning_step_llama3-8b_hbm_traffic.txt"),
+    ("llama2-7b-q100k", False): (49.984e9, "profiles/spanning_step_llama2-7b-q100k_hbm_traffic.txt"),
 }
 
 
