@@ -130,3 +130,36 @@ def test_row_cuts_cache_survives_route_changes_and_reloads(oracle):
             assert np.array_equal(got, oparams[i]), ctx
             if s + 1 in (1, 6, 10, 21, 24, 27):
                 assert_state_equal(opt.state[p], oref.state[i], ctx)
+
+
+def test_long_block_rows_with_heavy_ties_at_the_threshold(oracle):
+    """Rows of 1024 entries per block are selected from flags and the previous row's threshold
+    (hint_sorted_topk_bf16).  Gradients that take a handful of distinct magnitudes put hundreds
+    of equal keys at the threshold: which of them belong to the top-k is decided by coordinate,
+    and every row must be the oracle's, entry for entry."""
+    from ista_daslab_optimizers import MicroAdam
+    d = 20480 * 3
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    start = (torch.randn(d, generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+    oparams = [to_np(start).reshape(-1)]
+    oref = oracle.OracleMicroAdam(oparams, 20, 1e-3, 32, 0.05, 0.0, d_block_size=20480)
+    p = torch.nn.Parameter(start.clone())
+    opt = MicroAdam([p], m=20, lr=1e-3, quant_block_size=32, k_init=0.05, alpha=0.0)
+    levels = torch.tensor([1.0, 1.0, 1.0, 2.0, 2.0, 3.0, 4.0, 8.0], device="cuda") * 2 ** -10
+    ties = []
+    for s in range(8):
+        pick = torch.randint(0, 8, (d,), generator=gen, device="cuda")
+        sign = torch.randint(0, 2, (d,), generator=gen, device="cuda") * 2 - 1
+        g = (levels[pick] * sign).to(torch.bfloat16)
+        host = [to_np(g).reshape(-1)]
+        p.grad = g
+        opt.step()
+        oref.step(host)
+        assert opt._fusable(p, opt.state[p]) == 1
+        assert np.array_equal(to_np(p.data).reshape(-1), oparams[0]), f"step {s + 1}"
+        assert_state_equal(opt.state[p], oref.state[0], f"step {s + 1}")
+        V = opt.state[p]["V"][(opt.state[p]["index"] - 1) % 20, :1024].float().abs()
+        ties.append(int((V == V.min()).sum()))
+    # the case is what it claims: in rows written with a hint at hand (from the second step on)
+    # many entries share the smallest magnitude
+    assert max(ties[1:]) > 20, ties
