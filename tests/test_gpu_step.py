@@ -69,11 +69,13 @@ CASES = [
     ([32768 + 1000], torch.bfloat16, 3, 128, 0.01, 0.0, 0.0, 32768, 5),
     ([10240 * 2 + 8], torch.bfloat16, 3, 8, 0.01, 0.0, 0.0, 10240, 5),
     ([1001, 777], torch.bfloat16, 3, 64, 0.03, 0.0, 0.0, 20480, 5),   # odd d: partial chunks
-    # windows too large for the one-pass stage (20 rows of 5 %): the general stage, with the
-    # window held in registers (even k), streamed (odd k; more rows than the registers hold)
+    # windows too large for the one-pass stage (20 rows of 5 %): the step in two launches, the
+    # rows' chunk cuts cached; with weight decay and a tensor of exactly one block; more rows;
+    # fp32 data (the general selection, fp32 parameters in the window kernel)
     ([20480 * 2 + 8192], torch.bfloat16, 20, 32, 0.05, 0.0, 0.0, 20480, 23),
     ([20480 * 2 + 4096, 20480], torch.bfloat16, 20, 64, 0.05, 0.0, 0.01, 20480, 22),
     ([20480 + 8192], torch.bfloat16, 24, 32, 0.05, 0.0, 0.0, 20480, 26),
+    ([20480 * 2 + 8192], torch.float32, 20, 32, 0.05, 0.0, 0.0, 20480, 22),
     # quantisation blocks longer than the 512 elements a wave holds per chunk
     ([20480 * 2 + 4096, 3000, 12288], torch.bfloat16, 4, 1024, 0.01, 0.0, 0.0, 20480, 6),
     ([20480 + 5000], torch.bfloat16, 10, 4096, 0.01, 0.0, 0.01, 20480, 12),
