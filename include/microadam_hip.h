@@ -157,7 +157,9 @@ typedef struct ma_hyper {
 
 /* The whole of update_step (MA:146-328) for alpha == 0, for a list of tensors, in one pass per
  * top-k block: a = g + Qinv(e); block top-k -> I[index], V[index]; residual -> new min/max
- * and 4-bit codes; window -> Adam direction; p update (with decoupled weight decay).  The
+ * and 4-bit codes; window -> Adam direction; p update (with decoupled weight decay).  (Tensors
+ * whose window is about as dense as the tensor take two launches, the second for the window and
+ * the parameters: see ma_fused_step_row_cuts.)  The
  * caller advances st['index'] (MA:211) itself.  Conditions (else MA_ERR_NOT_FUSABLE, nothing
  * launched): quant_block_size a power of two in [8, 4096] that divides d_block_size (or
  * d <= d_block_size) and does not exceed d; p and g 16-byte aligned, error 4-byte aligned;
