@@ -76,6 +76,9 @@ CASES = [
     ([20480 * 2 + 4096, 20480], torch.bfloat16, 20, 64, 0.05, 0.0, 0.01, 20480, 22),
     ([20480 + 8192], torch.bfloat16, 24, 32, 0.05, 0.0, 0.0, 20480, 26),
     ([20480 * 2 + 8192], torch.float32, 20, 32, 0.05, 0.0, 0.0, 20480, 22),
+    # more rows than the one-pass stage takes, but short block rows (1 %), which the fast
+    # selections do not list by coordinate: two launches, the window kernel's general form
+    ([20480 * 2 + 8192, 4096], torch.bfloat16, 18, 64, 0.01, 0.0, 0.0, 20480, 21),
     # quantisation blocks longer than the 512 elements a wave holds per chunk
     ([20480 * 2 + 4096, 3000, 12288], torch.bfloat16, 4, 1024, 0.01, 0.0, 0.0, 20480, 6),
     ([20480 + 5000], torch.bfloat16, 10, 4096, 0.01, 0.0, 0.01, 20480, 12),
