@@ -79,6 +79,9 @@ CASES = [
     # more rows than the one-pass stage takes, but short block rows (1 %), which the fast
     # selections do not list by coordinate: two launches, the window kernel's general form
     ([20480 * 2 + 8192, 4096], torch.bfloat16, 18, 64, 0.01, 0.0, 0.0, 20480, 21),
+    # a fifth of every block selected: a row has about 100 entries per 512 coordinates, more
+    # than the window kernel's 64 lanes take in one go
+    ([20480 * 2 + 4096], torch.bfloat16, 4, 64, 0.2, 0.0, 0.0, 20480, 7),
     # quantisation blocks longer than the 512 elements a wave holds per chunk
     ([20480 * 2 + 4096, 3000, 12288], torch.bfloat16, 4, 1024, 0.01, 0.0, 0.0, 20480, 6),
     ([20480 + 5000], torch.bfloat16, 10, 4096, 0.01, 0.0, 0.01, 20480, 12),
